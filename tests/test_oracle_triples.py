@@ -1,0 +1,138 @@
+"""Pins triple lists, encodings and offsets (oracle/triples.py and cgnet_amd/CGutils.py) against
+closed-form counts, the parameter shapes the reference records, and the scipy MST fixture."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from oracle import triples as T
+from cgnet_amd import CGutils
+from cgnet_amd.CGutils import SparseLtuples as S
+
+
+def closed_form_count(lmax):
+    return sum(1 for l1 in range(lmax + 1) for l2 in range(l1 + 1) for l in range(lmax + 1)
+               if l1 - l2 <= l <= l1 + l2)
+
+
+@pytest.mark.parametrize("lmax,count", [(3, 23), (11, 489), (15, 1124), (20, 2486)])
+def test_default_counts(lmax, count):
+    assert closed_form_count(lmax) == count
+    codes, first = T.encode_sorted(T.default_pairs(lmax))
+    assert len(codes) == count
+    llls, table = S.sparse_rep_ltuples_sorted(S.compute_default_ltuples(lmax))
+    assert llls == codes
+    assert np.array_equal(table, first)
+    trip = S.get_iter(lmax, llls)
+    assert trip == T.decode(lmax, codes)
+    # ordered by l, then l1 ascending, l1 >= l2, triangle rule
+    assert trip == sorted(trip, key=lambda t: (t[0], t[1]))
+    assert all(l1 >= l2 and l1 - l2 <= l <= l1 + l2 for l, l1, l2 in trip)
+    # lookup table: first triple of degree l with l1 >= a
+    tab = table.reshape(lmax + 1, lmax + 2)
+    for l in range(lmax + 1):
+        for a in range(lmax + 2):
+            want = next((i for i, t in enumerate(trip) if t[0] > l or (t[0] == l and t[1] >= a)), len(trip))
+            assert tab[l, a] == want
+
+
+def test_config3_sizes():
+    lmax, tau = 11, [12] * 12
+    codes, _ = T.encode_sorted(T.default_pairs(lmax))
+    t_ff, t_off = T.product_taus(lmax, codes, tau)
+    assert t_ff == [1728, 3168, 4464, 5472, 6336, 6912, 7344, 7488, 7488, 7200, 6768, 6048]
+    assert T.cumulative_tm(tau)[-1] == 1728
+    assert T.cumulative_tm(t_ff)[-1] == 958032
+    assert sum(t_ff) == 70416
+    assert T.cumulative_w(t_ff, tau)[-1] == 844992
+    assert T.cg_table_offsets(lmax, codes)[-1] == 75625
+    assert t_ff == CGutils.calc_prod_taus(lmax, tau)
+    # offsets are the running channel count inside each degree
+    run = [0] * (lmax + 1)
+    for (l, l1, l2), off in zip(T.decode(lmax, codes), t_off):
+        assert off == run[l]
+        run[l] += tau[l1] * tau[l2]
+
+
+def test_reference_recorded_parameter_shapes():
+    # MNIST/example.sh:12 of the reference records W shapes (1643, 2) and (31023, 2) x 4 for
+    # "--lmax 11" (degrees 0..10), tau_type 3, tau_man 12, first layer fed with tau = 1.
+    lmax = 10
+    taus = [int(math.ceil(12 / math.sqrt(2 * l + 1.0))) for l in range(lmax + 1)]
+    codes, _ = T.encode_sorted(T.default_pairs(lmax))
+    t_ff0, _ = T.product_taus(lmax, codes, [1] * (lmax + 1))
+    t_ff1, _ = T.product_taus(lmax, codes, taus)
+    assert T.cumulative_w(t_ff0, taus)[-1] == 1643
+    assert T.cumulative_w(t_ff1, taus)[-1] == 31023
+    # embedding length 2 * sum of tau[0] over layers = 122 (BatchNorm1d(122) in the same record)
+    assert 2 * (1 + 5 * taus[0]) == 122
+
+
+@pytest.mark.parametrize("lmax", [3, 4, 8, 11, 15, 20])
+def test_mst_matches_scipy_fixture(golden_dir, lmax):
+    with open(os.path.join(golden_dir, "mst_scipy.json")) as fh:
+        fix = json.load(fh)["lmax"][str(lmax)]
+    want = [[tuple(p) for p in per_l] for per_l in fix]
+    assert T.mst_pairs(lmax, use_scipy=False) == want
+    assert S.compute_mst_ltuples(lmax) == want
+    for l in range(lmax + 1):
+        l1s, l2s = CGutils.compute_MST(l, lmax, diag=True)
+        assert list(zip(l1s, l2s)) == want[l]
+        t1, t2 = CGutils.compute_MST(l, lmax, diag=False)
+        assert list(zip(t1, t2)) == [p for p in want[l] if p[0] != p[1]]
+
+
+@pytest.mark.parametrize("lmax,count", [(11, 229), (15, 417), (20, 731)])
+def test_mst_properties(lmax, count):
+    pairs = T.mst_pairs(lmax, use_scipy=True)
+    assert sum(len(p) for p in pairs) == count
+    for l, per_l in enumerate(pairs):
+        edges = [(a, b) for a, b in per_l if a != b]
+        allowed = T.mst_edges(l, lmax)
+        nodes = {x for _, b, a in allowed for x in (a, b)}
+        # a spanning forest: acyclic, connects every node that has an edge
+        parent = {n: n for n in nodes}
+
+        def find(x):
+            while parent[x] != x:
+                x = parent[x]
+            return x
+        for a, b in edges:
+            assert a > b and a - b <= l <= a + b
+            ra, rb = find(a), find(b)
+            assert ra != rb
+            parent[ra] = rb
+        comps_tree = len({find(n) for n in nodes})
+        parent = {n: n for n in nodes}
+        for _, b, a in allowed:
+            ra, rb = find(a), find(b)
+            if ra != rb:
+                parent[ra] = rb
+        assert comps_tree == len({find(n) for n in nodes})
+        # minimal total weight: compare with scipy's tree weight
+        w = lambda a, b: (2 * l + 1) * (2 * a + 1) * (2 * b + 1)
+        assert sum(w(a, b) for a, b in edges) == sum(w(a, b) for a, b in T.mst_pairs_kruskal(l, lmax, False))
+
+
+def test_debug_and_user_lists():
+    assert S.compute_debug_ltuples(3) == T.debug_pairs(3)
+    assert all(len(p) <= 2 for p in S.compute_debug_ltuples(5))
+    with pytest.raises(AssertionError):
+        S.sparse_rep_ltuples_sorted([[(0, 1)], []])
+    # stable sort by l1 keeps the given l2 order
+    llls, _ = S.sparse_rep_ltuples_sorted([[(2, 2), (1, 1), (0, 0)], [(2, 1), (1, 0), (2, 2), (1, 1)], []])
+    assert S.get_iter(2, llls) == [(0, 0, 0), (0, 1, 1), (0, 2, 2), (1, 1, 0), (1, 1, 1), (1, 2, 1), (1, 2, 2)]
+
+
+def test_reshape_out_roundtrip():
+    import torch
+    taus = [2, 0, 3]
+    x = torch.arange(2 * (2 + 0 + 15) * 2, dtype=torch.float32).reshape(2, 17, 2)
+    parts = CGutils.reshape_out(x, taus)
+    assert [tuple(p.shape) for p in parts] == [(2, 2, 1, 2), (2, 0, 3, 2), (2, 3, 5, 2)]
+    assert torch.equal(torch.cat([p.reshape(2, -1, 2) for p in parts], 1), x)
+    assert parts[2].data_ptr() == x[:, 2:, :].data_ptr()            # a view, not a copy
+    with pytest.raises(AssertionError):
+        CGutils.reshape_out(x, [2, 1, 3])
