@@ -1,0 +1,58 @@
+"""Stack of Clebsch-Gordan layers with the l=0 skip-connection embedding: the reference's
+``SphericalCNN`` (CGNet/CGNet.py:14-69) on top of the HIP-backed ``CGBN_cuda`` layers."""
+import torch
+from torch import nn
+
+from . import CG_layers as cglayers
+
+
+class SphericalCNN(nn.Module):
+    def __init__(self, lmax, taus, cuda=True, norm=True, skipconn=True, sparse_flag=False, device=None):
+        """
+        :param lmax: degrees l = 0..lmax
+        :param taus: list of lists; taus[i] are the channels per degree entering layer i,
+            taus[i+1] the channels leaving it
+        :param cuda: must be True (the layers only run on the GPU)
+        :param norm: fragment normalisation on/off
+        :param skipconn: concatenate the l=0 fragments of the input and of every layer output;
+            otherwise only the last layer's l=0 fragment is returned
+        :param sparse_flag: True selects the minimum-spanning-tree subset of (l1, l2) pairs
+        :param device: overrides the device implied by ``cuda`` (e.g. 'cpu' to inspect parameters)
+        """
+        assert cuda, "Do not support these parameters yet"
+        super().__init__()
+        self.lmax = lmax
+        self.taus = taus
+        self.n_layers = len(taus) - 1
+        dev = 'cuda' if device is None else device
+        self.cgs = nn.ModuleList([cglayers.CGBN_cuda(lmax, taus[i], taus[i + 1], batchnorm=norm,
+                                                     sparse_flag=sparse_flag, device=dev)
+                                  for i in range(self.n_layers)])
+        self.skipconn = skipconn
+        if self.skipconn:
+            self.output_length = 2 * sum(int(t[0]) for t in taus)
+        else:
+            self.output_length = 2 * int(taus[-1][0])
+        self.to(dev)
+
+    def forward(self, f_input):
+        if isinstance(f_input, (list, tuple)):
+            B = f_input[0].shape[0]
+            first = f_input[0].reshape(B, -1)
+        else:
+            B = f_input.shape[0]
+            first = f_input[:, 0:int(self.taus[0][0]), :].reshape(B, -1)
+        embedding = [first] if self.skipconn else []
+        fs = f_input
+        for layer in self.cgs:
+            fs = layer(fs, straight_output=False)
+            if self.skipconn:
+                embedding.append(fs[0].reshape(B, -1))
+        if self.skipconn:
+            return torch.cat(embedding, 1)
+        return fs[0].reshape(B, -1)
+
+
+# The reference's README and Shrec17 script name a "SphericalCNN_fast"; its source is not part
+# of the reference, so only the name can be honoured.
+SphericalCNN_fast = SphericalCNN

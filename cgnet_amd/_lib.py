@@ -1,0 +1,78 @@
+"""ctypes binding of libcgnet_hip.so (C ABI declared in include/cgnet_hip.h).
+
+The library is built in-tree by ``make -C cgnet_amd/csrc`` (``__graft_entry__.build()``).
+There is no fallback: if the shared object is missing every operation raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libcgnet_hip.so")
+
+OK, ERR_ARG, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED = 0, -1, -2, -3, -4
+FN_BATCHNORM, FN_UPDATE_STD = 0x1, 0x2
+
+_c_int_p = ctypes.POINTER(ctypes.c_int)
+_vp = ctypes.c_void_p
+
+# name -> (restype, argtypes); the single source for the binding and for the symbol test
+SIGNATURES = {
+    "cgnet_last_error": (ctypes.c_char_p, []),
+    "cgnet_abi_version": (ctypes.c_int, []),
+    "cgnet_sparse_maxL": (ctypes.c_int, []),
+    "cgnet_sparse_precomputeCG": (ctypes.c_int, [_vp, ctypes.c_int, _c_int_p, ctypes.c_int, _c_int_p, _vp]),
+    "cgnet_cg_plan_create": (ctypes.c_int, [ctypes.POINTER(_vp), ctypes.c_int, _c_int_p, _c_int_p, ctypes.c_int,
+                                            _c_int_p, _c_int_p]),
+    "cgnet_cg_plan_destroy": (ctypes.c_int, [_vp]),
+    "cgnet_cg_plan_sizes": (ctypes.c_int, [_vp, _c_int_p]),
+    "cgnet_cg_plan_channels": (ctypes.c_int, [_vp, _c_int_p, _c_int_p]),
+    "cgnet_sparse_forward": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp]),
+    "cgnet_sparse_forward_stats_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_sparse_forward_stats": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_sparse_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_sparse_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_wmm_plan_create": (ctypes.c_int, [ctypes.POINTER(_vp), ctypes.c_int, _c_int_p, _c_int_p]),
+    "cgnet_wmm_plan_destroy": (ctypes.c_int, [_vp]),
+    "cgnet_wmm_plan_sizes": (ctypes.c_int, [_vp, _c_int_p]),
+    "cgnet_FN_WMM_forward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_FN_WMM_forward": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float, ctypes.c_float,
+                                            ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_FN_WMM_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_FN_WMM_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
+                                             ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+}
+
+_lib = None
+
+
+class CgnetError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("libcgnet_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+def load():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("%s is missing: build it with `make -C cgnet_amd/csrc` "
+                           "(or __graft_entry__.build()); there is no CPU fallback" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code):
+    if code != OK:
+        raise CgnetError(code, load().cgnet_last_error().decode("utf-8", "replace"))
+
+
+def int_array(values):
+    values = [int(v) for v in values]
+    return (ctypes.c_int * max(1, len(values)))(*values)

@@ -1,0 +1,697 @@
+// Fragment norm + per-degree complex channel mixing, forward and backward, for gfx950.
+//
+// The mixing of one degree l is a tall-skinny complex matrix product
+//     O[b, to, m] = sum_c  W[to, c] / div[c] * FF[b, c, m]        (t_O x t_FF) . (t_FF x (2l+1))
+// bounded by the one pass over FF.  It runs on the fp32 matrix cores as a real product with
+// twice the rows:  P = [W_re; W_im] . X  where X is FF with (re, im) as adjacent real columns;
+// then O_re = P_re-rows[re col] - P_im-rows[im col],  O_im = P_re-rows[im col] + P_im-rows[re col].
+//
+// v_mfma_f32_16x16x4_f32 operand layout (lane = 0..63): A[i][k] and B[k][j] sit in lane 16*k + i
+// (resp. 16*k + j); D[4*(lane/16) + v][lane%16] is register v of the lane.  The k slots and the
+// column slots of a tile can be assigned to memory freely as long as both operands agree, which
+// is used here so that every lane reads whole complex numbers (8-byte loads):
+//   forward : lane (k-slot kk, col-slot i) owns complex columns 2i and 2i+1 of a 32-column
+//             chunk; their (re, im) parts feed four column tiles.
+//   grad W  : the contraction runs over (b, m, re/im); lane (kk, i) reads complex entries
+//             8*blk + 2*kk, +1 of channel row i and feeds four k-steps.
+#include <algorithm>
+#include <memory>
+#include <vector>
+
+#include "common.h"
+
+namespace cgnet {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct WmmDeg {
+    int l, M;          // degree, 2l+1
+    int K, tO;         // mid channels, output channels
+    int cumFF, cumO;   // complex offsets of the degree inside a sample's FF / O
+    int cumW;          // complex offset of the degree's weights
+    int cumT;          // first mid channel of the degree among all mid channels
+    int nrc;           // row chunks of 16 output channels
+    int wp_base;       // first 64-float block of the degree in the packed weights
+    int G, NC;         // forward: samples per work-group, 32-column chunks per wave
+    int S;             // forward: number of k-slices
+};
+
+struct WmmFwdUnit { int deg, rc, slice, k_begin, k_end; };
+struct WmmChanUnit { int deg, rc, c0, nc; };   // a chunk of mid channels of one degree
+
+}  // namespace cgnet
+
+struct cgnet_wmm_plan {
+    int L = 0;
+    int nFF = 0, nO = 0, nW = 0, sumT = 0;
+    int wp_blocks = 0;     // 64-float blocks of the packed forward weights
+    int maxS = 1, maxG = 1;
+    std::vector<cgnet::WmmDeg> degs;
+    std::vector<cgnet::WmmFwdUnit> fwd_units;
+    std::vector<cgnet::WmmChanUnit> gw_units, gff_units, stat_units;
+    std::vector<int> cumO_all, cumFF_all;   // L+2 entries, for element -> degree lookups
+    cgnet::WmmDeg* d_degs = nullptr;
+    cgnet::WmmFwdUnit* d_fwd_units = nullptr;
+    cgnet::WmmChanUnit* d_gw_units = nullptr;
+    cgnet::WmmChanUnit* d_gff_units = nullptr;
+    cgnet::WmmChanUnit* d_stat_units = nullptr;
+    int* d_cumO = nullptr;      // per deg index: cumO, and S, interleaved: [ndeg+1] cumO then [ndeg] S
+    size_t stat_lds = 0, gff_lds = 0;
+};
+
+namespace cgnet {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kStatTileBytes = 32 * 1024;
+constexpr int kStatGroups = 8;
+
+// --------------------------------------------------------------------------- statistics
+// sums of |z| and |z|^2 over (b, m) per mid channel, from FF
+__global__ void __launch_bounds__(kThreads)
+fn_stats_kernel(const float2* __restrict__ FF, const WmmDeg* __restrict__ degs,
+                const WmmChanUnit* __restrict__ units, int nFF, int B, int samples_per_group,
+                double* __restrict__ part, int sumT) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float2* tile = reinterpret_cast<float2*>(smem);
+    const WmmChanUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    const int n = u.nc * d.M;
+    const int tid = threadIdx.x;
+    double s1 = 0., s2 = 0.;
+    const int b0 = blockIdx.y * samples_per_group, b1 = min(B, b0 + samples_per_group);
+    for (int b = b0; b < b1; ++b) {
+        const float2* src = FF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * d.M;
+        for (int e = tid; e < n; e += kThreads) tile[e] = src[e];
+        __syncthreads();
+        if (tid < u.nc) {
+            float a = 0.f, q = 0.f;
+            for (int mm = 0; mm < d.M; ++mm) {
+                const float2 z = tile[tid * d.M + mm];
+                const float nn = fmaf(z.x, z.x, z.y * z.y);
+                q += nn;
+                a += sqrtf(nn);
+            }
+            s1 += (double)a;
+            s2 += (double)q;
+        }
+        __syncthreads();
+    }
+    if (tid < u.nc) {
+        double* p = part + ((size_t)blockIdx.y * sumT + d.cumT + u.c0 + tid) * 2;
+        p[0] = s1;
+        p[1] = s2;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+fn_sum_groups_kernel(const double* __restrict__ part, double* __restrict__ sums, int n2, int ngroups) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n2) return;
+    double s = 0.;
+    for (int g = 0; g < ngroups; ++g) s += part[(size_t)g * n2 + i];
+    sums[i] = s;
+}
+
+// stds[c] <- stds[c] * cnt/(cnt+1) + std_batch[c] / (cnt+1)
+__global__ void __launch_bounds__(256)
+fn_update_std_kernel(const double* __restrict__ sums, float* __restrict__ stds,
+                     const WmmDeg* __restrict__ degs, int ndeg, int sumT, int B, float cnt) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= sumT) return;
+    int di = 0;
+    while (di + 1 < ndeg && degs[di + 1].cumT <= c) ++di;
+    const double N = (double)B * (double)degs[di].M;
+    const double mean = sums[2 * c] / N;
+    double var = sums[2 * c + 1] / N - mean * mean;
+    const double sd = var > 0. ? sqrt(var) : 0.;
+    float m = stds[c];
+    m *= cnt / (cnt + 1.f);
+    m = (float)((double)m + sd / (double)(cnt + 1.f));
+    stds[c] = m;
+}
+
+// --------------------------------------------------------------------------- weight packing
+// Forward operand: for every degree, k-step ks (4 channels), row chunk rc: two 64-lane blocks
+// (rows = W_re, rows = W_im), lane 16*kk + row holds W[rc*16+row][4*ks+kk] / div.
+__global__ void __launch_bounds__(256)
+pack_w_forward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                      const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int total_blocks) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int blk = idx >> 6, lane = idx & 63;
+    if (blk >= total_blocks) return;
+    int di = 0;
+    while (di + 1 < ndeg && degs[di + 1].wp_base <= blk) ++di;
+    const WmmDeg d = degs[di];
+    const int rel = blk - d.wp_base;             // ((ks * nrc) + rc) * 2 + tile
+    const int tile = rel & 1;
+    const int rc = (rel >> 1) % d.nrc;
+    const int ks = (rel >> 1) / d.nrc;
+    const int row = lane & 15, kk = lane >> 4;
+    const int to = rc * 16 + row, c = ks * 4 + kk;
+    float v = 0.f;
+    if (to < d.tO && c < d.K) {
+        const float2 w = W[d.cumW + (size_t)to * d.K + c];
+        v = tile ? w.y : w.x;
+        if (stds) v /= fmaxf(eps, stds[d.cumT + c]);
+    }
+    Wp[idx] = v;
+}
+
+// Backward operand: WT[cumW + c*tO + to] = conj(W[to][c]) / div[c]
+__global__ void __launch_bounds__(256)
+pack_w_backward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                       const WmmDeg* __restrict__ degs, int ndeg, float2* __restrict__ WT, int nW) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= nW) return;
+    int di = 0;
+    while (di + 1 < ndeg && degs[di + 1].cumW <= idx) ++di;
+    const WmmDeg d = degs[di];
+    const int rel = idx - d.cumW;
+    const int c = rel / d.tO, to = rel % d.tO;
+    float2 w = W[d.cumW + (size_t)to * d.K + c];
+    float r = 1.f;
+    if (stds) r = fmaxf(eps, stds[d.cumT + c]);
+    WT[idx] = make_float2(w.x / r, -w.y / r);
+}
+
+// --------------------------------------------------------------------------- forward (MFMA)
+__device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+template <int NC>
+__device__ __forceinline__ void wmm_forward_body(const float* __restrict__ FF, const float* __restrict__ Wp,
+                                                 float2* __restrict__ out, const WmmDeg& d,
+                                                 const WmmFwdUnit& u, int B, int nFF, int nO, f32x4 (*red)[8][64]) {
+    const int b0 = blockIdx.y * d.G;
+    if (b0 >= B) return;
+    const int nb = min(d.G, B - b0);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int i = lane & 15, kk = lane >> 4;
+    const int M = d.M, n2 = 2 * d.M;
+    const int ncols = nb * M;
+
+    size_t off[NC][2];
+    bool ok[NC][2];
+#pragma unroll
+    for (int nc = 0; nc < NC; ++nc)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int q = nc * 32 + 2 * i + h;
+            ok[nc][h] = q < ncols;
+            const int bl = ok[nc][h] ? q / M : 0;
+            const int m = ok[nc][h] ? q - bl * M : 0;
+            off[nc][h] = ((size_t)(b0 + bl) * nFF + d.cumFF + m) * 2;
+        }
+
+    f32x4 acc[2][NC * 4];
+#pragma unroll
+    for (int t = 0; t < NC * 4; ++t) {
+        acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        acc[1][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    const int nsteps = (u.k_end - u.k_begin + 3) >> 2;
+    const int ks0 = u.k_begin >> 2;
+    for (int s = w; s < nsteps; s += 4) {
+        const int k = u.k_begin + 4 * s + kk;
+        const bool kin = k < u.k_end;
+        const float* ap = Wp + ((size_t)(d.wp_base + ((ks0 + s) * d.nrc + u.rc) * 2)) * 64 + lane;
+        const float a0 = ap[0], a1 = ap[64];
+        float2 bv[NC][2];
+#pragma unroll
+        for (int nc = 0; nc < NC; ++nc)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                bv[nc][h] = make_float2(0.f, 0.f);
+                if (ok[nc][h] && kin) bv[nc][h] = *reinterpret_cast<const float2*>(FF + off[nc][h] + (size_t)k * n2);
+            }
+#pragma unroll
+        for (int nc = 0; nc < NC; ++nc) {
+            acc[0][nc * 4 + 0] = mfma4(a0, bv[nc][0].x, acc[0][nc * 4 + 0]);
+            acc[0][nc * 4 + 1] = mfma4(a0, bv[nc][0].y, acc[0][nc * 4 + 1]);
+            acc[0][nc * 4 + 2] = mfma4(a0, bv[nc][1].x, acc[0][nc * 4 + 2]);
+            acc[0][nc * 4 + 3] = mfma4(a0, bv[nc][1].y, acc[0][nc * 4 + 3]);
+            acc[1][nc * 4 + 0] = mfma4(a1, bv[nc][0].x, acc[1][nc * 4 + 0]);
+            acc[1][nc * 4 + 1] = mfma4(a1, bv[nc][0].y, acc[1][nc * 4 + 1]);
+            acc[1][nc * 4 + 2] = mfma4(a1, bv[nc][1].x, acc[1][nc * 4 + 2]);
+            acc[1][nc * 4 + 3] = mfma4(a1, bv[nc][1].y, acc[1][nc * 4 + 3]);
+        }
+    }
+
+    // add the four waves' partial sums in a fixed order, then form the complex outputs
+    float2* dst = out + (size_t)u.slice * B * nO;
+#pragma unroll
+    for (int nc = 0; nc < NC; ++nc) {
+        __syncthreads();
+        if (w > 0) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                red[w - 1][t][lane] = acc[0][nc * 4 + t];
+                red[w - 1][4 + t][lane] = acc[1][nc * 4 + t];
+            }
+        }
+        __syncthreads();
+        if (w == 0) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc[0][nc * 4 + t] = ((acc[0][nc * 4 + t] + red[0][t][lane]) + red[1][t][lane]) + red[2][t][lane];
+                acc[1][nc * 4 + t] = ((acc[1][nc * 4 + t] + red[0][4 + t][lane]) + red[1][4 + t][lane]) + red[2][4 + t][lane];
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (!ok[nc][h]) continue;
+                const int q = nc * 32 + 2 * i + h;
+                const int bl = q / M, m = q - bl * M;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int to = u.rc * 16 + 4 * kk + v;
+                    if (to < d.tO) {
+                        const float re = acc[0][nc * 4 + 2 * h][v] - acc[1][nc * 4 + 2 * h + 1][v];
+                        const float im = acc[0][nc * 4 + 2 * h + 1][v] + acc[1][nc * 4 + 2 * h][v];
+                        dst[(size_t)(b0 + bl) * nO + d.cumO + to * M + m] = make_float2(re, im);
+                    }
+                }
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kThreads)
+wmm_forward_kernel(const float* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
+                   const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO) {
+    __shared__ f32x4 red[3][8][64];
+    const WmmFwdUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    switch (d.NC) {
+        case 1: wmm_forward_body<1>(FF, Wp, out, d, u, B, nFF, nO, red); break;
+        case 2: wmm_forward_body<2>(FF, Wp, out, d, u, B, nFF, nO, red); break;
+        default: wmm_forward_body<3>(FF, Wp, out, d, u, B, nFF, nO, red); break;
+    }
+}
+
+// O = sum over k-slices of the partial outputs, in slice order
+__global__ void __launch_bounds__(256)
+wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
+                      const int* __restrict__ cumO_S, int ndeg, int B, int nO) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)B * nO) return;
+    const int e = (int)(idx % nO);
+    int di = 0;
+    while (di + 1 < ndeg && cumO_S[di + 1] <= e) ++di;
+    const int S = cumO_S[ndeg + 1 + di];
+    float2 s = part[idx];
+    for (int k = 1; k < S; ++k) {
+        const float2 v = part[(size_t)k * B * nO + idx];
+        s.x += v.x;
+        s.y += v.y;
+    }
+    O[idx] = s;
+}
+
+// --------------------------------------------------------------------------- grad W (MFMA)
+__global__ void __launch_bounds__(kThreads)
+wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, const float* __restrict__ stds,
+                 float eps, float2* __restrict__ gW, const WmmDeg* __restrict__ degs,
+                 const WmmChanUnit* __restrict__ units, int B, int nFF, int nO) {
+    const WmmChanUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int i = lane & 15, kk = lane >> 4;
+    const int M = d.M;
+    const int c = u.c0 + 16 * w + i;          // B operand: mid channel of this lane
+    const bool cok = c < d.K && (16 * w + i) < u.nc;
+    const int to_a = u.rc * 16 + i;           // A operand: output channel of this lane
+    const bool tok = to_a < d.tO;
+    const int nblk = (M + 7) >> 3;
+    const size_t f_row = (size_t)d.cumFF + (size_t)(cok ? c : 0) * M;
+    const size_t g_row = (size_t)d.cumO + (size_t)(tok ? to_a : 0) * M;
+
+    f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < B; ++b) {
+        const float2* frow = FF + (size_t)b * nFF + f_row;
+        const float2* grow = gO + (size_t)b * nO + g_row;
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int p0 = blk * 8 + kk * 2;
+            float2 f0 = make_float2(0.f, 0.f), f1 = f0, g0 = f0, g1 = f0;
+            if (p0 < M) {
+                if (cok) f0 = frow[p0];
+                if (tok) g0 = grow[p0];
+            }
+            if (p0 + 1 < M) {
+                if (cok) f1 = frow[p0 + 1];
+                if (tok) g1 = grow[p0 + 1];
+            }
+            acc0 = mfma4(g0.x, f0.x, acc0);
+            acc0 = mfma4(g0.y, f0.y, acc0);
+            acc0 = mfma4(g1.x, f1.x, acc0);
+            acc0 = mfma4(g1.y, f1.y, acc0);
+            acc1 = mfma4(g0.y, f0.x, acc1);
+            acc1 = mfma4(-g0.x, f0.y, acc1);
+            acc1 = mfma4(g1.y, f1.x, acc1);
+            acc1 = mfma4(-g1.x, f1.y, acc1);
+        }
+        if ((b & 7) == 7) {
+            tot0 += acc0;
+            tot1 += acc1;
+            acc0 = (f32x4){0.f, 0.f, 0.f, 0.f};
+            acc1 = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    tot0 += acc0;
+    tot1 += acc1;
+    if (cok) {
+        float r = 1.f;
+        if (stds) r = fmaxf(eps, stds[d.cumT + c]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int to = u.rc * 16 + 4 * kk + v;
+            if (to < d.tO) gW[d.cumW + (size_t)to * d.K + c] = make_float2(tot0[v] / r, tot1[v] / r);
+        }
+    }
+}
+
+// --------------------------------------------------------------------------- grad FF
+// gFF[b, c, m] = sum_to WT[c][to] * gO[b, to, m]   with WT = conj(W)/div packed channel-major
+__global__ void __launch_bounds__(kThreads)
+wmm_gradff_kernel(const float2* __restrict__ gO, const float2* __restrict__ WT, float2* __restrict__ gFF,
+                  const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int nFF, int nO) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float2* go = reinterpret_cast<float2*>(smem);      // [tO][M]
+    const WmmChanUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    const int b = blockIdx.y;
+    const int M = d.M, tO = d.tO;
+    const float2* src = gO + (size_t)b * nO + d.cumO;
+    for (int e = threadIdx.x; e < tO * M; e += kThreads) go[e] = src[e];
+    __syncthreads();
+    const int n = u.nc * M;
+    float2* dst = gFF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M;
+    for (int e = threadIdx.x; e < n; e += kThreads) {
+        const int cl = e / M, m = e - cl * M;
+        const float2* wt = WT + d.cumW + (size_t)(u.c0 + cl) * tO;
+        float re = 0.f, im = 0.f;
+        for (int to = 0; to < tO; ++to) {
+            const float2 wv = wt[to];
+            const float2 gv = go[to * M + m];
+            re = fmaf(wv.x, gv.x, re);
+            re = fmaf(-wv.y, gv.y, re);
+            im = fmaf(wv.x, gv.y, im);
+            im = fmaf(wv.y, gv.x, im);
+        }
+        dst[e] = make_float2(re, im);
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(float* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+int stat_groups_for(int B) { return std::max(1, std::min(B, kStatGroups)); }
+
+struct FwdWorkspace {
+    size_t sums, part, wp, opart, total;
+};
+
+FwdWorkspace fwd_workspace(const cgnet_wmm_plan* p, int B) {
+    FwdWorkspace w;
+    size_t o = 0;
+    w.sums = o;
+    o += align_up(sizeof(double) * 2 * (size_t)p->sumT, 256);
+    w.part = o;
+    o += align_up(sizeof(double) * 2 * (size_t)p->sumT * stat_groups_for(B), 256);
+    w.wp = o;
+    o += align_up(sizeof(float) * 64 * (size_t)p->wp_blocks, 256);
+    w.opart = o;
+    if (p->maxS > 1) o += align_up(sizeof(float) * 2 * (size_t)p->nO * B * p->maxS, 256);
+    w.total = o;
+    return w;
+}
+
+}  // namespace
+}  // namespace cgnet
+
+using namespace cgnet;
+
+static void free_plan(cgnet_wmm_plan* plan) {
+    if (!plan) return;
+    void* ptrs[] = {plan->d_degs, plan->d_fwd_units, plan->d_gw_units, plan->d_gff_units, plan->d_stat_units, plan->d_cumO};
+    for (void* q : ptrs)
+        if (q) (void)hipFree(q);
+    delete plan;
+}
+
+extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_t_FF, const int* h_t_O) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    *plan = nullptr;
+    CGNET_REQUIRE(L >= 0 && L <= kMaxL, CGNET_ERR_UNSUPPORTED, "lmax=%d outside [0, %d]", L, kMaxL);
+    CGNET_REQUIRE(h_t_FF && h_t_O, CGNET_ERR_ARG, "null pointer argument");
+    cgnet_wmm_plan* p = new cgnet_wmm_plan();
+    std::unique_ptr<cgnet_wmm_plan, void (*)(cgnet_wmm_plan*)> guard(p, free_plan);
+    p->L = L;
+    long long cFF = 0, cO = 0, cW = 0, cT = 0;
+    int wp = 0;
+    for (int l = 0; l <= L; ++l) {
+        const int K = h_t_FF[l], tO = h_t_O[l], M = 2 * l + 1;
+        CGNET_REQUIRE(K >= 0 && tO >= 0, CGNET_ERR_ARG, "negative channel count at degree %d", l);
+        CGNET_REQUIRE(tO <= kMaxTau, CGNET_ERR_UNSUPPORTED, "t_O[%d]=%d above %d", l, tO, kMaxTau);
+        WmmDeg d;
+        d.l = l; d.M = M; d.K = K; d.tO = tO;
+        d.cumFF = (int)cFF; d.cumO = (int)cO; d.cumW = (int)cW; d.cumT = (int)cT;
+        d.nrc = std::max(1, (tO + 15) / 16);
+        d.wp_base = wp;
+        // forward: G samples x M complex columns per wave in NC chunks of 32 columns
+        int bestG = 1, bestNC = (M + 31) / 32;
+        if (M <= 96) {
+            double best = -1;
+            for (int nc = 1; nc <= 3; ++nc) {
+                const int g = (32 * nc) / M;
+                if (g < 1) continue;
+                const double eff = (double)g * M / (32.0 * nc);
+                if (eff > best + 1e-9) { best = eff; bestG = g; bestNC = nc; }
+            }
+        }
+        d.G = bestG;
+        d.NC = bestNC;
+        // k-slices of about 1024 channels (multiples of 4)
+        d.S = std::max(1, (K + 1023) / 1024);
+        p->degs.push_back(d);
+        cFF += (long long)K * M;
+        cO += (long long)tO * M;
+        cW += (long long)K * tO;
+        cT += K;
+        wp += ((K + 3) / 4) * d.nrc * 2;
+        CGNET_REQUIRE(cFF < (1LL << 30) && cW < (1LL << 30), CGNET_ERR_UNSUPPORTED, "sizes above 2^30 complex entries");
+    }
+    p->nFF = (int)cFF; p->nO = (int)cO; p->nW = (int)cW; p->sumT = (int)cT;
+    p->wp_blocks = wp;
+    const int ndeg = (int)p->degs.size();
+    for (int di = 0; di < ndeg; ++di) {
+        const WmmDeg& d = p->degs[di];
+        if (d.K == 0 || d.tO == 0) continue;
+        CGNET_REQUIRE(d.NC <= 3, CGNET_ERR_UNSUPPORTED, "degree %d has more than 96 columns per sample", d.l);
+        p->maxS = std::max(p->maxS, d.S);
+        p->maxG = std::max(p->maxG, d.G);
+        const int steps = (d.K + 3) / 4;
+        const int per = ((steps + d.S - 1) / d.S) * 4;
+        for (int rc = 0; rc < d.nrc; ++rc)
+            for (int s = 0; s < d.S; ++s) {
+                WmmFwdUnit u{di, rc, s, std::min(d.K, s * per), std::min(d.K, (s + 1) * per)};
+                p->fwd_units.push_back(u);
+            }
+        for (int rc = 0; rc < d.nrc; ++rc)
+            for (int c0 = 0; c0 < d.K; c0 += 64) p->gw_units.push_back(WmmChanUnit{di, rc, c0, std::min(64, d.K - c0)});
+    }
+    for (int di = 0; di < ndeg; ++di) {
+        const WmmDeg& d = p->degs[di];
+        if (d.K == 0) continue;
+        const int per_stat = std::max(1, std::min(kThreads, kStatTileBytes / (8 * d.M)));
+        for (int c0 = 0; c0 < d.K; c0 += per_stat)
+            p->stat_units.push_back(WmmChanUnit{di, 0, c0, std::min(per_stat, d.K - c0)});
+        p->stat_lds = std::max(p->stat_lds, (size_t)8 * per_stat * d.M);
+        const int per_gff = std::max(1, 4096 / d.M);
+        for (int c0 = 0; c0 < d.K; c0 += per_gff)
+            p->gff_units.push_back(WmmChanUnit{di, 0, c0, std::min(per_gff, d.K - c0)});
+        p->gff_lds = std::max(p->gff_lds, (size_t)8 * d.tO * d.M);
+    }
+    CGNET_REQUIRE(p->gff_lds <= 64 * 1024, CGNET_ERR_UNSUPPORTED, "t_O*(2l+1) too large for the gradient kernel");
+    // heavier forward units first
+    std::stable_sort(p->fwd_units.begin(), p->fwd_units.end(), [&](const WmmFwdUnit& a, const WmmFwdUnit& b) {
+        return (long long)(a.k_end - a.k_begin) * p->degs[a.deg].M > (long long)(b.k_end - b.k_begin) * p->degs[b.deg].M;
+    });
+    std::stable_sort(p->gw_units.begin(), p->gw_units.end(), [&](const WmmChanUnit& a, const WmmChanUnit& b) {
+        return p->degs[a.deg].M > p->degs[b.deg].M;
+    });
+
+    std::vector<int> cumO_S(2 * ndeg + 1);
+    for (int di = 0; di < ndeg; ++di) cumO_S[di] = p->degs[di].cumO;
+    cumO_S[ndeg] = p->nO;
+    for (int di = 0; di < ndeg; ++di) cumO_S[ndeg + 1 + di] = (p->degs[di].K == 0 || p->degs[di].tO == 0) ? 0 : p->degs[di].S;
+
+    auto upload = [&](const void* src, size_t bytes, void** dst) -> int {
+        if (bytes == 0) return CGNET_OK;
+        CGNET_HIP(hipMalloc(dst, bytes));
+        CGNET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return CGNET_OK;
+    };
+    int rc;
+    if ((rc = upload(p->degs.data(), sizeof(WmmDeg) * ndeg, (void**)&p->d_degs))) return rc;
+    if ((rc = upload(p->fwd_units.data(), sizeof(WmmFwdUnit) * p->fwd_units.size(), (void**)&p->d_fwd_units))) return rc;
+    if ((rc = upload(p->gw_units.data(), sizeof(WmmChanUnit) * p->gw_units.size(), (void**)&p->d_gw_units))) return rc;
+    if ((rc = upload(p->gff_units.data(), sizeof(WmmChanUnit) * p->gff_units.size(), (void**)&p->d_gff_units))) return rc;
+    if ((rc = upload(p->stat_units.data(), sizeof(WmmChanUnit) * p->stat_units.size(), (void**)&p->d_stat_units))) return rc;
+    if ((rc = upload(cumO_S.data(), sizeof(int) * cumO_S.size(), (void**)&p->d_cumO))) return rc;
+    *plan = guard.release();
+    return CGNET_OK;
+}
+
+extern "C" int cgnet_wmm_plan_destroy(cgnet_wmm_plan* plan) {
+    clear_error();
+    free_plan(plan);
+    return CGNET_OK;
+}
+
+extern "C" int cgnet_wmm_plan_sizes(const cgnet_wmm_plan* plan, int sizes[4]) {
+    clear_error();
+    CGNET_REQUIRE(plan && sizes, CGNET_ERR_ARG, "null pointer argument");
+    sizes[0] = plan->nFF;
+    sizes[1] = plan->nO;
+    sizes[2] = plan->nW;
+    sizes[3] = plan->sumT;
+    return CGNET_OK;
+}
+
+extern "C" size_t cgnet_FN_WMM_forward_workspace(const cgnet_wmm_plan* plan, int B) {
+    if (!plan || B <= 0) return 0;
+    return fwd_workspace(plan, B).total;
+}
+
+extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_FF, float* d_O, const float* d_W,
+                                    int B, float* d_stds, float cnt, float eps, int flags, const double* d_sums,
+                                    void* d_workspace, size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    if (B == 0) return CGNET_OK;
+    const bool bn = flags & CGNET_FN_BATCHNORM, upd = bn && (flags & CGNET_FN_UPDATE_STD);
+    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    CGNET_REQUIRE(plan->nO == 0 || d_O, CGNET_ERR_ARG, "d_O is NULL");
+    CGNET_REQUIRE(plan->nFF == 0 || d_FF, CGNET_ERR_ARG, "d_FF is NULL");
+    CGNET_REQUIRE(plan->nW == 0 || d_W, CGNET_ERR_ARG, "d_W is NULL");
+    const FwdWorkspace ws = fwd_workspace(plan, B);
+    CGNET_REQUIRE(d_workspace && workspace_bytes >= ws.total, CGNET_ERR_WORKSPACE,
+                  "workspace of %zu bytes given, %zu needed", workspace_bytes, ws.total);
+    hipStream_t s = (hipStream_t)stream;
+    char* base = (char*)d_workspace;
+    const int ndeg = (int)plan->degs.size();
+
+    if (upd && plan->sumT > 0) {
+        const double* sums = d_sums;
+        if (!sums) {
+            const int ng = stat_groups_for(B);
+            const int spg = (B + ng - 1) / ng;
+            const int ngroups = (B + spg - 1) / spg;
+            hipLaunchKernelGGL(fn_stats_kernel, dim3((unsigned)plan->stat_units.size(), ngroups), dim3(kThreads),
+                               plan->stat_lds, s, (const float2*)d_FF, plan->d_degs, plan->d_stat_units, plan->nFF,
+                               B, spg, (double*)(base + ws.part), plan->sumT);
+            CGNET_HIP(hipGetLastError());
+            const int n2 = 2 * plan->sumT;
+            hipLaunchKernelGGL(fn_sum_groups_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
+                               (const double*)(base + ws.part), (double*)(base + ws.sums), n2, ngroups);
+            CGNET_HIP(hipGetLastError());
+            sums = (const double*)(base + ws.sums);
+        }
+        hipLaunchKernelGGL(fn_update_std_kernel, dim3((plan->sumT + 255) / 256), dim3(256), 0, s, sums, d_stds,
+                           plan->d_degs, ndeg, plan->sumT, B, cnt);
+        CGNET_HIP(hipGetLastError());
+    }
+    if (plan->nO == 0) return CGNET_OK;
+    if (plan->fwd_units.empty()) {   // degrees with outputs but no mid channels produce zeros
+        const size_t n = (size_t)2 * plan->nO * B;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_O, n);
+        CGNET_HIP(hipGetLastError());
+        return CGNET_OK;
+    }
+    float* Wp = (float*)(base + ws.wp);
+    const int total = plan->wp_blocks * 64;
+    hipLaunchKernelGGL(pack_w_forward_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
+                       bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Wp, plan->wp_blocks);
+    CGNET_HIP(hipGetLastError());
+    // degrees with t_O > 0 but no mid channels are never written by the product kernel
+    bool holes = false;
+    for (const WmmDeg& d : plan->degs) holes |= (d.tO > 0 && d.K == 0);
+    float2* out = plan->maxS > 1 ? (float2*)(base + ws.opart) : (float2*)d_O;
+    if (holes || plan->maxS > 1) {
+        const size_t n = (size_t)2 * plan->nO * B * (plan->maxS > 1 ? plan->maxS : 1);
+        if (holes) {
+            hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)out, n);
+            CGNET_HIP(hipGetLastError());
+        }
+    }
+    int ygroups = 1;
+    for (const WmmDeg& d : plan->degs)
+        if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + d.G - 1) / d.G);
+    CGNET_REQUIRE(ygroups <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d too large", B);
+    hipLaunchKernelGGL(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads), 0, s,
+                       d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO);
+    CGNET_HIP(hipGetLastError());
+    if (plan->maxS > 1) {
+        const size_t n = (size_t)plan->nO * B;
+        hipLaunchKernelGGL(wmm_sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+                           (const float2*)out, (float2*)d_O, plan->d_cumO, ndeg, B, plan->nO);
+        CGNET_HIP(hipGetLastError());
+    }
+    return CGNET_OK;
+}
+
+extern "C" size_t cgnet_FN_WMM_backward_workspace(const cgnet_wmm_plan* plan, int B) {
+    if (!plan || B <= 0) return 0;
+    return align_up(sizeof(float) * 2 * (size_t)plan->nW, 256);
+}
+
+extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* d_gFF, float* d_gW,
+                                     const float* d_FF, const float* d_W, int B, const float* d_stds, float eps,
+                                     int flags, void* d_workspace, size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    const bool bn = flags & CGNET_FN_BATCHNORM;
+    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    const int ndeg = (int)plan->degs.size();
+    if (d_gW && plan->nW > 0) {
+        if (B == 0 || plan->nO == 0) {
+            const size_t n = (size_t)2 * plan->nW;
+            hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gW, n);
+            CGNET_HIP(hipGetLastError());
+        } else {
+            CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
+            hipLaunchKernelGGL(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size()), dim3(kThreads), 0, s,
+                               (const float2*)d_gO, (const float2*)d_FF, bn ? d_stds : nullptr, eps, (float2*)d_gW,
+                               plan->d_degs, plan->d_gw_units, B, plan->nFF, plan->nO);
+            CGNET_HIP(hipGetLastError());
+        }
+    }
+    if (d_gFF && plan->nFF > 0 && B > 0) {
+        CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
+        CGNET_REQUIRE(d_W, CGNET_ERR_ARG, "d_W is NULL");
+        CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
+        const size_t need = cgnet_FN_WMM_backward_workspace(plan, B);
+        CGNET_REQUIRE(d_workspace && workspace_bytes >= need, CGNET_ERR_WORKSPACE,
+                      "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+        float2* WT = (float2*)d_workspace;
+        if (plan->nW > 0) {
+            hipLaunchKernelGGL(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
+                               (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
+            CGNET_HIP(hipGetLastError());
+        }
+        hipLaunchKernelGGL(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
+                           plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
+                           plan->d_gff_units, plan->nFF, plan->nO);
+        CGNET_HIP(hipGetLastError());
+    }
+    return CGNET_OK;
+}

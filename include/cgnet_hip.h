@@ -1,0 +1,144 @@
+/*
+ * cgnet_hip.h -- C ABI of libcgnet_hip.so: the Clebsch-Gordan layer hot path on MI355X (gfx950).
+ *
+ * Every entry point takes plain pointers and sizes.  Device pointers are marked d_, host
+ * pointers h_.  `stream` is a hipStream_t passed as void* (NULL = the default stream); work
+ * is enqueued on it and the call returns without synchronising the device.  Return value:
+ * CGNET_OK or a negative CGNET_ERR_* code; cgnet_last_error() then holds a message for the
+ * calling thread.  The caller owns every buffer, outputs included (as in the reference, where
+ * the Python side allocates outputs and the native side fills them in place).
+ *
+ * Each function names the reference interface it stands in for.  File:line citations are
+ * relative to the reference checkout (zlin7/CGNet).  The reference binds these operations
+ * through the pybind11 module `CG_cuda_ops` (CGNet/cudaCG/cudaCG_all.cpp:207-215); that
+ * module passes int32 device tensors for the per-degree metadata, which forces the kernels to
+ * re-derive the layout on every call.  Here the metadata is handed over once, from host
+ * arrays, into a plan object; the per-call functions then take only data pointers.
+ *
+ * Tensor layouts (all float32, complex numbers interleaved (re, im)):
+ *   "straight" fragments  F  [B][nF ][2], nF  = sum_l t_F [l](2l+1); inside degree l: [t][m]
+ *   CG product            FF [B][nFF][2], nFF = sum_l t_FF[l](2l+1)
+ *   layer output          O  [B][nO ][2], nO  = sum_l t_O [l](2l+1)
+ *   weights               W  [nW][2], nW = sum_l t_O[l]*t_FF[l]; degree l is a row-major
+ *                            (t_O[l], t_FF[l]) complex matrix
+ *   CG table              CG [cg_len]; triple i owns (2l+1)(2l2+1) floats at CG_offsets[i],
+ *                            entry [m+l][m2+l2] = <l1 m-m2 l2 m2 | l m>, 0 where |m-m2| > l1
+ */
+#ifndef CGNET_HIP_H
+#define CGNET_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CGNET_OK               0
+#define CGNET_ERR_ARG         (-1)   /* null pointer, negative size, inconsistent metadata */
+#define CGNET_ERR_HIP         (-2)   /* a HIP runtime call failed */
+#define CGNET_ERR_WORKSPACE   (-3)   /* workspace missing or smaller than *_workspace() */
+#define CGNET_ERR_UNSUPPORTED (-4)   /* size beyond what the kernels are built for */
+
+/* fragment-norm flags of FN_WMM_forward / FN_WMM_backward (CGNet/CG_layers.py:22-33) */
+#define CGNET_FN_BATCHNORM   0x1     /* divide each mid channel by max(eps, std) */
+#define CGNET_FN_UPDATE_STD  0x2     /* fold this batch into the running stds before use */
+
+typedef struct cgnet_cg_plan  cgnet_cg_plan;
+typedef struct cgnet_wmm_plan cgnet_wmm_plan;
+
+/* Message describing the last error on the calling thread ("" if none). */
+const char* cgnet_last_error(void);
+
+/* ABI revision of this header. */
+int cgnet_abi_version(void);
+
+/* Largest supported lmax.  Replaces CG_cuda_ops.sparse_maxL (cudaCG_all.cpp:130-132). */
+int cgnet_sparse_maxL(void);
+
+/* Fill the flat Clebsch-Gordan table on the device (double-precision Racah sum, stored as
+ * float).  Replaces CG_cuda_ops.sparse_precomputeCG (cudaCG_all.cpp:114-127; kernel
+ * cudaCG_sparse.cu:68-92, host :304-317).  h_llls[i] = (l*(L+1)+l1)*(L+1)+l2 with l1 >= l2;
+ * h_CG_offsets has nllls+1 entries.  Every entry of the table is written (zeros included). */
+int cgnet_sparse_precomputeCG(float* d_CG, int L, const int* h_llls, int nllls,
+                              const int* h_CG_offsets, void* stream);
+
+/* ---- Clebsch-Gordan product ------------------------------------------------------------ */
+
+/* Build the plan of one CG product: h_t_F[L+1] input channels per degree, h_llls[nllls] kept
+ * triples in the order that fixes the output channel order.  h_t_offsets (nllls entries,
+ * channel offset of each triple inside its output degree) and h_CG_offsets (nllls+1) may be
+ * NULL, in which case they are the running sums the reference computes at
+ * CGNet/CG_layers.py:253-262 and CGNet/CGutils.py:179-187.  Stands in for the int32 device
+ * tensors t_F, cumu_tm_F, t_FF, cumu_tm_FF, llls, l_l1_to_lllidx_offsets, t_offsets,
+ * CG_offsets that the reference passes on every call (cudaCG_all.cpp:39-51). */
+int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_F, const int* h_llls, int nllls,
+                         const int* h_t_offsets, const int* h_CG_offsets);
+int cgnet_cg_plan_destroy(cgnet_cg_plan* plan);
+/* sizes[0..4] = nF, nFF, sum_l t_FF[l], cg_len, nllls */
+int cgnet_cg_plan_sizes(const cgnet_cg_plan* plan, int sizes[5]);
+/* h_t_FF[L+1], h_t_offsets[nllls]; either may be NULL */
+int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, int* h_t_offsets);
+
+/* FF = CG product of F with itself over the plan's triples:
+ *   FF[b, l, t_off + t1*t_F[l2] + t2, m] = sum_{m1+m2=m} CG * F[b,l1,t1,m1] * F[b,l2,t2,m2].
+ * Replaces CG_cuda_ops.sparse_forward (cudaCG_all.cpp:39-71; kernel cudaCG_sparse.cu:96-184).
+ * Every element of d_FF is written; it need not be zeroed. */
+int cgnet_sparse_forward(const cgnet_cg_plan* plan, const float* d_F, float* d_FF,
+                         const float* d_CG, int B, void* stream);
+
+/* Same product that also returns, per mid channel c, sum_{b,m} |FF| and sum_{b,m} |FF|^2 in
+ * d_sums[2*c], d_sums[2*c+1] (double), so that the fragment-norm statistics need no second
+ * pass over FF.  No counterpart in the reference (its statistics kernel
+ * cudaCG_FNWMM.cu:29-79 re-reads FF); the result feeds cgnet_FN_WMM_forward(d_sums=...). */
+size_t cgnet_sparse_forward_stats_workspace(const cgnet_cg_plan* plan, int B);
+int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float* d_F, float* d_FF,
+                               const float* d_CG, int B, double* d_sums,
+                               void* d_workspace, size_t workspace_bytes, void* stream);
+
+/* Gradient of the product with respect to F given d_gFF = dLoss/dFF:
+ *   gF[b,l1,t1,m1] = sum CG * gFF[b,l,t,m1+m2] * conj(F[b,l2,t2,m2])  + the same with the
+ *   roles of the two slots exchanged (a diagonal triple l1 == l2 contributes through both).
+ * Replaces CG_cuda_ops.sparse_backward (cudaCG_all.cpp:73-108; kernel cudaCG_sparse.cu:186-298).
+ * Deterministic.  Every element of d_gF is written. */
+size_t cgnet_sparse_backward_workspace(const cgnet_cg_plan* plan, int B);
+int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F, float* d_gF,
+                          const float* d_gFF, const float* d_CG, int B,
+                          void* d_workspace, size_t workspace_bytes, void* stream);
+
+/* ---- fragment norm + per-degree complex weight mixing -------------------------------- */
+
+/* Plan for mixing h_t_FF[l] mid channels into h_t_O[l] output channels, l = 0..L.  Stands in
+ * for the device tensors t_FF, cumu_tm_FF, t_O, cumu_tm_O, cumu_tt_W (cudaCG_all.cpp:137-146). */
+int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_t_FF, const int* h_t_O);
+int cgnet_wmm_plan_destroy(cgnet_wmm_plan* plan);
+/* sizes[0..3] = nFF, nO, nW, sum_l t_FF[l] */
+int cgnet_wmm_plan_sizes(const cgnet_wmm_plan* plan, int sizes[4]);
+
+/* O[b,l,to,m] = sum_c W[l,to,c] * FF[b,l,c,m] / max(eps, stds[c])   (no division without
+ * CGNET_FN_BATCHNORM).  With CGNET_FN_UPDATE_STD the running stds are first updated in place:
+ *   s = population std over (b, m) of |FF[b,l,c,m]|;  stds[c] = stds[c]*cnt/(cnt+1) + s/(cnt+1)
+ * and the updated value normalises this very batch.  d_sums, if not NULL, holds the per-channel
+ * sums produced by cgnet_sparse_forward_stats and replaces the statistics pass over FF.
+ * Replaces CG_cuda_ops.FN_WMM_forward (cudaCG_all.cpp:137-165; kernels cudaCG_FNWMM.cu:29-123,
+ * host :215-245).  d_stds may be NULL when CGNET_FN_BATCHNORM is not set. */
+size_t cgnet_FN_WMM_forward_workspace(const cgnet_wmm_plan* plan, int B);
+int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_FF, float* d_O, const float* d_W,
+                         int B, float* d_stds, float cnt, float eps, int flags, const double* d_sums,
+                         void* d_workspace, size_t workspace_bytes, void* stream);
+
+/* gW[l,to,c]   = sum_{b,m} gO[b,l,to,m] * conj(FF[b,l,c,m]) / max(eps, stds[c])
+ * gFF[b,l,c,m] = (sum_to conj(W[l,to,c]) * gO[b,l,to,m]) / max(eps, stds[c])
+ * with the stds treated as constants.  Replaces CG_cuda_ops.FN_WMM_backward
+ * (cudaCG_all.cpp:172-205; kernels cudaCG_FNWMM.cu:126-211, host :250-282).  Unlike the
+ * reference (float atomics over the batch) the gW reduction is deterministic.  Every element
+ * of d_gFF and d_gW is written.  Either of d_gFF / d_gW may be NULL to skip that output. */
+size_t cgnet_FN_WMM_backward_workspace(const cgnet_wmm_plan* plan, int B);
+int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* d_gFF, float* d_gW,
+                          const float* d_FF, const float* d_W, int B, const float* d_stds,
+                          float eps, int flags,
+                          void* d_workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CGNET_HIP_H */

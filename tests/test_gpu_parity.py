@@ -1,0 +1,447 @@
+"""GPU parity tests: every native entry point against the CPU oracle on the same seeded inputs.
+
+Tolerance (the north star's fp32 bar): |gpu - oracle64| <= 1e-6 * max(1, rms(oracle64)) + 1e-5 * |oracle64|
+elementwise, where oracle64 is the float64 evaluation of the reference's python algorithm.  The
+absolute term is expressed in units of the tensor's RMS once that exceeds 1, because float32
+cannot resolve 1e-6 on values of magnitude >> 1 (weight gradients reach ~1e2).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cg_coeff as OC
+from oracle import cg_layer as OL
+from oracle import triples as OT
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU: torch.cuda.is_available() is False")
+    from cgnet_amd import _lib
+    _lib.load()                      # raises if the HIP library was not built
+    return torch.device("cuda:0")
+
+
+def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
+    got = got.detach().double().cpu().reshape(-1)
+    ref = ref.detach().double().cpu().reshape(-1)
+    assert got.shape == ref.shape, what
+    assert torch.isfinite(got).all(), what + ": non-finite values"
+    rms = float(ref.pow(2).mean().sqrt()) if ref.numel() else 0.0
+    bound = atol * max(1.0, rms) + rtol * ref.abs()
+    err = (got - ref).abs()
+    worst = int(torch.argmax(err - bound)) if ref.numel() else 0
+    assert bool((err <= bound).all()), (
+        "%s: %d of %d outside tolerance; worst |err|=%.3e at %d (ref %.6e, bound %.3e, rms %.3e)"
+        % (what, int((err > bound).sum()), ref.numel(), float(err[worst]), worst, float(ref[worst]),
+           float(bound[worst]), rms))
+
+
+def make_codes(lmax, mode):
+    if mode == "default":
+        pairs = OT.default_pairs(lmax)
+    elif mode == "mst":
+        pairs = OT.mst_pairs(lmax, use_scipy=False)
+    elif mode == "debug":
+        pairs = OT.debug_pairs(lmax)
+    else:
+        pairs = mode
+    return OT.encode_sorted(pairs)[0]
+
+
+def rand_straight(taus, bsz, seed, scaled=True):
+    g = torch.Generator().manual_seed(seed)
+    parts = []
+    for l, t in enumerate(taus):
+        x = torch.randn(bsz, t * (2 * l + 1), 2, generator=g, dtype=torch.float64)
+        parts.append(x / math.sqrt(2 * l + 1) if scaled else x)
+    return torch.cat(parts, dim=1)
+
+
+# ------------------------------------------------------------------------------- CG table
+@pytest.mark.parametrize("lmax,mode", [(3, "default"), (11, "default"), (15, "mst"), (20, "default"), (5, "debug")])
+def test_cg_table_matches_oracle(dev, lmax, mode):
+    from cgnet_amd import CG_cuda_ops
+    codes = make_codes(lmax, mode)
+    want, offs = OC.flat_cg_table(OT.decode(lmax, codes), dtype=np.float64)
+    cg = torch.full((int(offs[-1]),), float("nan"), device=dev)
+    CG_cuda_ops.sparse_precomputeCG(cg, lmax, torch.tensor(codes, dtype=torch.int32, device=dev),
+                                    torch.tensor(offs, dtype=torch.int32, device=dev))
+    got = cg.cpu().double().numpy()
+    assert np.isfinite(got).all()
+    assert np.max(np.abs(got - want)) <= 1.2e-7          # float32 rounding of values <= 1
+    assert np.array_equal(got == 0, np.abs(want) < 1e-30) or np.max(np.abs(got[np.abs(want) < 1e-30])) == 0
+
+
+# ------------------------------------------------------------------------------- CG product
+CG_CASES = [
+    # lmax, taus, B, mode
+    (3, [2, 2, 2, 2], 4, "default"),                      # BASELINE config 1
+    (3, [2, 2, 2, 2], 4, "mst"),
+    (4, [3, 1, 0, 5, 2], 3, "default"),                   # ragged, a degree without channels
+    (2, [1, 1, 1], 1, "default"),                         # tau = 1 everywhere, single sample
+    (5, [7, 6, 5, 13, 3, 9], 5, "mst"),
+    (6, [17, 4, 4, 4, 4, 4, 33], 2, "debug"),             # more than 16 channels in the reduced slot
+    (11, [5] * 12, 6, "default"),                         # BASELINE config 2 shape, small batch
+    (11, [12] * 12, 3, "default"),                        # BASELINE config 3 shape, small batch
+    (15, [16] * 16, 2, "mst"),                            # BASELINE config 4 shape, small batch
+]
+
+
+def cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64=None):
+    x = x64.clone().requires_grad_(True)
+    y = OL.join_straight(OL.cg_product(x, lmax, codes, taus))
+    if gy64 is None:
+        return y.detach(), None
+    (gx,) = torch.autograd.grad(y, x, gy64)
+    return y.detach(), gx
+
+
+@pytest.mark.parametrize("lmax,taus,bsz,mode", CG_CASES)
+def test_cg_forward_backward(dev, lmax, taus, bsz, mode):
+    from cgnet_amd import CG_layers
+    codes = make_codes(lmax, mode)
+    x64 = rand_straight(taus, bsz, seed=lmax * 100 + bsz)
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, lll_mode=None if mode == "default" else mode, device=dev)
+    assert mod.lll_list == codes
+    g = torch.Generator().manual_seed(17)
+    gy64 = torch.randn(bsz, int(mod.cumu_tm_FF[-1]), 2, generator=g, dtype=torch.float64)
+    want_y, want_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64)
+
+    x = x64.float().to(dev).requires_grad_(True)
+    y = mod(x, straight_output=True)
+    assert y.shape == want_y.shape
+    assert_close(y, want_y, "CG forward")
+    y.backward(gy64.float().to(dev))
+    assert_close(x.grad, want_gx, "CG backward")
+
+    # list input / list output views
+    parts = OL.split_straight(x.detach(), taus)
+    y_list = mod([p.contiguous() for p in parts], straight_output=False)
+    assert [tuple(p.shape) for p in y_list] == [(bsz, int(t), 2 * l + 1, 2) for l, t in enumerate(mod.t_FF)]
+    assert torch.equal(torch.cat([p.reshape(bsz, -1, 2) for p in y_list], 1), y.detach())
+
+
+def test_cg_forward_matches_dense_definition(dev):
+    # config 1 against the explicit six-index loop definition (independent of the oracle's matmul path)
+    from oracle import bruteforce as BF
+    from cgnet_amd import CG_layers
+    lmax, taus, bsz = 3, [2, 2, 2, 2], 4
+    codes = make_codes(lmax, "default")
+    x64 = rand_straight(taus, bsz, seed=0, scaled=False)
+    fs = OL.split_straight(x64, taus)
+    want = BF.cg_product_loops([f[..., 0].numpy() + 1j * f[..., 1].numpy() for f in fs], OT.decode(lmax, codes), taus)
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, device=dev)
+    got = mod(x64.float().to(dev), straight_output=False)
+    for l in range(lmax + 1):
+        z = got[l].cpu().double()
+        z = z[..., 0].numpy() + 1j * z[..., 1].numpy()
+        assert np.max(np.abs(z - want[l])) <= 2e-6 * max(1.0, np.max(np.abs(want[l])))
+
+
+def test_cg_deterministic(dev):
+    from cgnet_amd import CG_layers
+    lmax, taus, bsz = 11, [12] * 12, 5
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, device=dev)
+    x = rand_straight(taus, bsz, 3).float().to(dev).requires_grad_(True)
+    gy = torch.randn(bsz, int(mod.cumu_tm_FF[-1]), 2, device=dev)
+    outs = []
+    for _ in range(2):
+        x.grad = None
+        y = mod(x)
+        y.backward(gy)
+        outs.append((y.detach().clone(), x.grad.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+# ------------------------------------------------------------------------------- fragment norm + mixing
+def wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds, eps, bn, training, cnt, go64=None):
+    ff = ff64.clone().requires_grad_(True)
+    w = w64.clone().requires_grad_(True)
+    parts = OL.split_straight(ff, t_ff)
+    st, o = [], 0
+    for t in t_ff:
+        st.append(np.array(stds[o:o + t], dtype=np.float64))
+        o += t
+    if bn:
+        OL.fragment_norm_update([p for p in parts], st, cnt, training)
+        parts = OL.fragment_normalise(parts, st, eps)
+    out = OL.join_straight(OL.weight_mix(parts, w, t_ff, t_out))
+    res = {"out": out.detach(), "stds": np.concatenate(st) if len(st) else np.zeros(0)}
+    if go64 is not None:
+        gff, gw = torch.autograd.grad(out, (ff, w), go64)
+        res["gFF"], res["gW"] = gff, gw
+    return res
+
+
+WMM_CASES = [
+    # lmax, t_FF, t_O, B, batchnorm, training
+    (3, [12, 20, 24, 16], [2, 2, 2, 2], 4, True, True),
+    (3, [12, 20, 24, 16], [2, 2, 2, 2], 4, True, False),
+    (3, [12, 20, 24, 16], [2, 2, 2, 2], 4, False, True),
+    (4, [5, 0, 9, 130, 7], [3, 2, 0, 17, 1], 5, True, True),     # empty degrees, t_O > 16, K not multiple of 4
+    (2, [1, 1, 1], [1, 1, 1], 1, True, True),
+    (11, [300, 500, 700, 900, 1100, 1200, 1300, 1300, 1300, 1250, 1180, 1050], [12] * 12, 9, True, True),
+    (20, [64] * 21, [16] * 21, 3, True, True),                    # 41 complex columns per sample
+]
+
+
+@pytest.mark.parametrize("lmax,t_ff,t_out,bsz,bn,training", WMM_CASES)
+def test_fn_wmm_forward_backward(dev, lmax, t_ff, t_out, bsz, bn, training):
+    from cgnet_amd import CG_layers
+    g = torch.Generator().manual_seed(1000 + lmax + bsz)
+    ff64 = rand_straight(t_ff, bsz, seed=5) * 0.3
+    n_w = sum(a * b for a, b in zip(t_ff, t_out))
+    w64 = torch.cat([torch.randn(t_ff[l] * t_out[l], 2, generator=g, dtype=torch.float64) / math.sqrt(max(1, t_ff[l]))
+                     for l in range(lmax + 1)]) if n_w else torch.zeros(0, 2, dtype=torch.float64)
+    stds0 = (0.05 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64) * 0.3).float()
+    if sum(t_ff) > 3:
+        stds0[1] = 1e-9                                   # exercises the eps floor
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(t_out))
+    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
+    cnt = 3.0
+    want = wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds0.double().numpy(), 1e-5, bn, training, cnt, go64)
+
+    mod = CG_layers.MyBatchNormWeightMM_cuda(lmax, t_ff, t_out, batchnorm=bn, device=dev)
+    with torch.no_grad():
+        mod.W.copy_(w64.float())
+        if bn:
+            mod.bn_stds.copy_(stds0)
+    mod.bn_cnt = cnt
+    mod.train(training)
+    ff = ff64.float().to(dev).requires_grad_(True)
+    out = mod(ff)
+    assert out.shape == (bsz, n_o, 2)
+    assert_close(out, want["out"], "WMM forward")
+    if bn:
+        assert_close(mod.bn_stds, torch.from_numpy(want["stds"]), "running stds", rtol=2e-6, atol=1e-8)
+        assert mod.bn_cnt == (cnt + 1 if training else cnt)
+    out.backward(go64.float().to(dev))
+    assert_close(ff.grad, want["gFF"], "grad FF")
+    assert_close(mod.W.grad, want["gW"], "grad W")
+
+
+def test_gradw_deterministic(dev):
+    from cgnet_amd import CG_layers
+    lmax, t_ff, t_out, bsz = 5, [40, 64, 100, 130, 90, 70], [6] * 6, 13
+    mod = CG_layers.MyBatchNormWeightMM_cuda(lmax, t_ff, t_out, device=dev)
+    mod.eval()
+    ff = rand_straight(t_ff, bsz, 2).float().to(dev)
+    go = torch.randn(bsz, int(mod.cumu_tm_O[-1]), 2, device=dev)
+    grads = []
+    for _ in range(2):
+        mod.W.grad = None
+        mod(ff).backward(go)
+        grads.append(mod.W.grad.clone())
+    assert torch.equal(grads[0], grads[1])
+
+
+# ------------------------------------------------------------------------------- whole layer and stack
+LAYER_CASES = [
+    # lmax, taus_in, taus_out, B, sparse_flag, batchnorm
+    (3, [2, 2, 2, 2], [2, 2, 2, 2], 4, False, True),
+    (3, [2, 2, 2, 2], [3, 1, 2, 2], 4, True, True),
+    (4, [3, 2, 1, 2, 2], [2, 2, 2, 2, 2], 3, False, False),
+    (11, [5] * 12, [5] * 12, 8, False, True),            # BASELINE config 2 shape (B reduced for the oracle)
+    (11, [12] * 12, [12] * 12, 3, False, True),          # BASELINE config 3 shape (B reduced)
+]
+
+
+def build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed):
+    from cgnet_amd import CG_layers
+    mod = CG_layers.CGBN_cuda(lmax, tin, tout, batchnorm=bn, sparse_flag=sparse, device=dev)
+    codes = mod.cg.lll_list
+    ora = OL.LayerOracle(lmax, tin, tout, codes, batchnorm=bn, eps=1e-5)
+    g = torch.Generator().manual_seed(seed)
+    t_ff = [int(v) for v in mod.t_FF]
+    w64 = torch.cat([torch.randn(t_ff[l] * tout[l], 2, generator=g, dtype=torch.float64) / math.sqrt(max(1, t_ff[l]))
+                     for l in range(lmax + 1)])
+    stds = 0.02 + 0.1 * torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
+    with torch.no_grad():
+        mod.bnWMM.W.copy_(w64.float())
+        if bn:
+            mod.bnWMM.bn_stds.copy_(stds.float())
+    if bn:
+        ora.set_stds_flat(stds.float().double().numpy())
+    return mod, ora, w64.float().double()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn", LAYER_CASES)
+def test_layer_forward_backward(dev, lmax, tin, tout, bsz, sparse, bn, fused):
+    mod, ora, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=lmax + bsz)
+    mod.fused = fused
+    x64 = rand_straight(tin, bsz, seed=21)
+    g = torch.Generator().manual_seed(23)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
+
+    xo = x64.float().double().requires_grad_(True)
+    wo = w64.clone().requires_grad_(True)
+    want = OL.join_straight(ora.forward(xo, wo))
+    want_gx, want_gw = torch.autograd.grad(want, (xo, wo), go64)
+
+    x = x64.float().to(dev).requires_grad_(True)
+    out = mod(x, straight_output=True)
+    assert_close(out, want, "layer forward")
+    if bn:
+        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds", rtol=5e-6, atol=1e-8)
+        assert mod.bnWMM.bn_cnt == 2.0
+    out.backward(go64.float().to(dev))
+    assert_close(x.grad, want_gx, "layer grad F")
+    assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W")
+
+    # second training step: the moving average advances with count 2
+    if bn:
+        want2 = OL.join_straight(ora.forward(xo.detach() * 0.5, wo.detach()))
+        out2 = mod((x.detach() * 0.5), straight_output=True)
+        assert_close(out2, want2, "second step forward")
+        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds step 2", rtol=5e-6, atol=1e-8)
+        # eval mode leaves the statistics alone
+        mod.eval()
+        ora.training = False
+        keep = mod.bnWMM.bn_stds.clone()
+        out3 = mod(x.detach(), straight_output=False)
+        want3 = ora.forward(xo.detach(), wo.detach())
+        assert torch.equal(keep, mod.bnWMM.bn_stds) and mod.bnWMM.bn_cnt == 3.0
+        for a, b in zip(out3, want3):
+            assert_close(a, b, "eval forward")
+
+
+def test_spherical_cnn_stack(dev):
+    from cgnet_amd import CGNet
+    lmax = 4
+    taus = [[1] * 5, [3] * 5, [2, 3, 2, 1, 2]]
+    net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
+    assert net.output_length == 2 * (1 + 3 + 2)
+    layers, ws = [], []
+    g = torch.Generator().manual_seed(3)
+    for i, cg in enumerate(net.cgs):
+        ora = OL.LayerOracle(lmax, taus[i], taus[i + 1], cg.cg.lll_list, batchnorm=True)
+        t_ff = [int(v) for v in cg.t_FF]
+        w64 = torch.randn(sum(a * b for a, b in zip(t_ff, taus[i + 1])), 2, generator=g, dtype=torch.float64) * 0.3
+        stds = 0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
+        with torch.no_grad():
+            cg.bnWMM.W.copy_(w64.float())
+            cg.bnWMM.bn_stds.copy_(stds.float())
+        ora.set_stds_flat(stds.float().double().numpy())
+        layers.append(ora)
+        ws.append(w64.float().double().requires_grad_(True))
+    # real-signal symmetry f_l^{-m} = (-1)^m conj(f_l^m)
+    bsz = 3
+    parts = []
+    for l in range(lmax + 1):
+        z = torch.randn(bsz, 1, 2 * l + 1, 2, generator=g, dtype=torch.float64)
+        for m in range(1, l + 1):
+            sign = (-1.0) ** m
+            z[:, :, l - m, 0] = sign * z[:, :, l + m, 0]
+            z[:, :, l - m, 1] = -sign * z[:, :, l + m, 1]
+        z[:, :, l, 1] = 0
+        parts.append(z.reshape(bsz, -1, 2))
+    x64 = torch.cat(parts, 1).float().double()
+    xo = x64.clone().requires_grad_(True)
+    want = OL.stack_forward(layers, ws, xo, taus[0], skipconn=True)
+    head = torch.randn(want.shape[1], 10, generator=g, dtype=torch.float64) * 0.2
+    labels = torch.randint(0, 10, (bsz,), generator=g)
+    loss_o = torch.nn.functional.cross_entropy(want @ head, labels)
+    grads_o = torch.autograd.grad(loss_o, [xo] + ws)
+
+    x = x64.float().to(dev).requires_grad_(True)
+    emb = net(x)
+    assert emb.shape == (bsz, net.output_length)
+    assert_close(emb, want, "stack embedding", rtol=2e-5, atol=2e-6)
+    loss = torch.nn.functional.cross_entropy(emb.double() @ head.to(dev), labels.to(dev))
+    loss.backward()
+    assert_close(x.grad, grads_o[0], "stack grad input", rtol=1e-4, atol=2e-6)
+    for i, cg in enumerate(net.cgs):
+        assert_close(cg.bnWMM.W.grad, grads_o[1 + i], "stack grad W%d" % i, rtol=1e-4, atol=2e-6)
+
+
+# ------------------------------------------------------------------------------- full-size properties
+def test_full_size_properties_config3(dev):
+    """BASELINE config 3 (L=11, tau=12, B=100): properties that need no CPU-sized oracle."""
+    from cgnet_amd import CG_layers
+    lmax, taus, bsz = 11, [12] * 12, 100
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, device=dev)
+    x = rand_straight(taus, bsz, 11).float().to(dev)
+    y = mod(x)
+    assert y.shape == (bsz, 958032, 2) and torch.isfinite(y).all()
+    # bilinearity
+    assert torch.allclose(mod(2 * x), 4 * y, rtol=1e-6, atol=1e-7)
+    # equivariance under a rotation about z: fragment m picks up exp(-i m alpha) on both sides
+    alpha = 0.37
+
+    def rotate(t, chans):
+        out = torch.empty_like(t)
+        o = 0
+        for l, c in enumerate(chans):
+            n = int(c) * (2 * l + 1)
+            ang = -alpha * torch.arange(-l, l + 1, device=t.device, dtype=torch.float64)
+            cs, sn = torch.cos(ang).float(), torch.sin(ang).float()
+            blk = t[:, o:o + n].reshape(t.shape[0], int(c), 2 * l + 1, 2)
+            re = blk[..., 0] * cs - blk[..., 1] * sn
+            im = blk[..., 0] * sn + blk[..., 1] * cs
+            out[:, o:o + n] = torch.stack([re, im], -1).reshape(t.shape[0], n, 2)
+            o += n
+        return out
+    assert torch.allclose(mod(rotate(x, taus)), rotate(y, mod.t_FF), rtol=1e-4, atol=2e-6)
+    # every sample is independent of its batch neighbours
+    y7 = mod(x[7:8].contiguous())
+    assert torch.equal(y7[0], y[7])
+    # adjoint identity <gy, J dx> = <J^T gy, dx> with J dx = CG(x+dx) - CG(x) - CG(dx)  (bilinear map)
+    dx = 1e-2 * torch.randn_like(x)
+    gy = torch.randn_like(y)
+    xr = x.clone().requires_grad_(True)
+    mod(xr).backward(gy)
+    jdx = (mod(x + dx) - y - mod(dx)).double()
+    lhs = float((gy.double() * jdx).sum())
+    rhs = float((xr.grad.double() * dx.double()).sum())
+    assert lhs == pytest.approx(rhs, rel=2e-4)
+
+
+def test_full_size_layer_config3_runs(dev):
+    from cgnet_amd import CG_layers
+    lmax, tau, bsz = 11, [12] * 12, 100
+    mod = CG_layers.CGBN_cuda(lmax, tau, tau, device=dev)
+    with torch.no_grad():
+        mod.bnWMM.W.normal_(0, 0.01)
+        mod.bnWMM.bn_stds.fill_(1.0)
+    x = rand_straight(tau, bsz, 4).float().to(dev).requires_grad_(True)
+    out = mod(x, straight_output=True)
+    assert out.shape == (bsz, 1728, 2)
+    out.backward(torch.randn_like(out))
+    assert torch.isfinite(out).all() and torch.isfinite(x.grad).all() and torch.isfinite(mod.bnWMM.W.grad).all()
+    # fused and unfused paths agree (same kernels except where the statistics are taken)
+    mod2 = CG_layers.CGBN_cuda(lmax, tau, tau, device=dev)
+    mod2.load_state_dict(mod.state_dict())
+    with torch.no_grad():
+        mod2.bnWMM.bn_stds.fill_(1.0)
+    mod2.fused = False
+    out2 = mod2(x.detach(), straight_output=True)
+    assert torch.allclose(out, out2, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(mod.bnWMM.bn_stds, mod2.bnWMM.bn_stds, rtol=1e-6, atol=1e-9)
+
+
+# ------------------------------------------------------------------------------- error behaviour
+def test_errors(dev):
+    from cgnet_amd import CG_cuda_ops, CG_layers, _plans
+    mod = CG_layers.CG_woFilter_cuda(2, [1, 1, 1], device=dev)
+    with pytest.raises(AssertionError):
+        mod(torch.zeros(1, 9, 2))                         # CPU tensor, as in the reference
+    with pytest.raises(RuntimeError):
+        mod(torch.zeros(1, 8, 2, device=dev))             # wrong number of input coefficients
+    with pytest.raises(RuntimeError):
+        _plans.CGPlan(2, [1, 1, 1], [5 * 9 + 1])          # l=0 from (l1=0, l2=... ) code violating l1 >= l2
+    with pytest.raises(RuntimeError):
+        _plans.CGPlan(99, [1] * 100, [])
+    assert CG_cuda_ops.sparse_maxL() >= 20
+    # empty batch is a no-op
+    y = mod(torch.zeros(0, 9, 2, device=dev))
+    assert y.shape[0] == 0
