@@ -65,6 +65,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kStatTileBytes = 32 * 1024;
 constexpr int kStatGroups = 8;
+constexpr int kGradWChunk = 32;     // samples accumulated in one matrix-core chain of the weight gradient
 
 // --------------------------------------------------------------------------- statistics
 // sums of |z| and |z|^2 over (b, m) per mid channel, from FF
@@ -180,6 +181,15 @@ __device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// Called between the last matrix instruction of a chain and the first ordinary read of its
+// accumulators: gives the matrix pipeline time to retire its results (an accumulator read
+// hoisted directly behind the chain returned stale values otherwise).
+__device__ __forceinline__ void mfma_drain() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int NC>
 __device__ __forceinline__ void wmm_forward_body(const float* __restrict__ FF, const float* __restrict__ Wp,
                                                  float2* __restrict__ out, const WmmDeg& d,
@@ -239,6 +249,7 @@ __device__ __forceinline__ void wmm_forward_body(const float* __restrict__ FF, c
         }
     }
 
+    mfma_drain();
     // add the four waves' partial sums in a fixed order, then form the complex outputs
     float2* dst = out + (size_t)u.slice * B * nO;
 #pragma unroll
@@ -310,10 +321,12 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
 }
 
 // --------------------------------------------------------------------------- grad W (MFMA)
+// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples (blockIdx.y)
+// into part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
 __global__ void __launch_bounds__(kThreads)
-wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, const float* __restrict__ stds,
-                 float eps, float2* __restrict__ gW, const WmmDeg* __restrict__ degs,
-                 const WmmChanUnit* __restrict__ units, int B, int nFF, int nO) {
+wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, float2* __restrict__ part,
+                 const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
+                 int samples_per_chunk, int nFF, int nO, int nW) {
     const WmmChanUnit u = units[blockIdx.x];
     const WmmDeg d = degs[u.deg];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -327,9 +340,10 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, c
     const size_t f_row = (size_t)d.cumFF + (size_t)(cok ? c : 0) * M;
     const size_t g_row = (size_t)d.cumO + (size_t)(tok ? to_a : 0) * M;
 
-    f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    for (int b = 0; b < B; ++b) {
+    const int b_begin = blockIdx.y * samples_per_chunk;
+    const int b_end = min(B, b_begin + samples_per_chunk);
+    for (int b = b_begin; b < b_end; ++b) {
         const float2* frow = FF + (size_t)b * nFF + f_row;
         const float2* grow = gO + (size_t)b * nO + g_row;
         for (int blk = 0; blk < nblk; ++blk) {
@@ -352,24 +366,39 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, c
             acc1 = mfma4(g1.y, f1.x, acc1);
             acc1 = mfma4(-g1.x, f1.y, acc1);
         }
-        if ((b & 7) == 7) {
-            tot0 += acc0;
-            tot1 += acc1;
-            acc0 = (f32x4){0.f, 0.f, 0.f, 0.f};
-            acc1 = (f32x4){0.f, 0.f, 0.f, 0.f};
-        }
     }
-    tot0 += acc0;
-    tot1 += acc1;
+    mfma_drain();
     if (cok) {
-        float r = 1.f;
-        if (stds) r = fmaxf(eps, stds[d.cumT + c]);
+        float2* dst = part + (size_t)blockIdx.y * nW;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int to = u.rc * 16 + 4 * kk + v;
-            if (to < d.tO) gW[d.cumW + (size_t)to * d.K + c] = make_float2(tot0[v] / r, tot1[v] / r);
+            if (to < d.tO) dst[d.cumW + (size_t)to * d.K + c] = make_float2(acc0[v], acc1[v]);
         }
     }
+}
+
+__global__ void __launch_bounds__(256)
+wmm_gradw_finish_kernel(const float2* __restrict__ part, const float* __restrict__ stds, float eps,
+                        const WmmDeg* __restrict__ degs, int ndeg, float2* __restrict__ gW, int nW, int nchunks) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= nW) return;
+    float2 s = part[idx];
+    for (int k = 1; k < nchunks; ++k) {
+        const float2 v = part[(size_t)k * nW + idx];
+        s.x += v.x;
+        s.y += v.y;
+    }
+    if (stds) {
+        int di = 0;
+        while (di + 1 < ndeg && degs[di + 1].cumW <= idx) ++di;
+        const WmmDeg d = degs[di];
+        const int c = (idx - d.cumW) % d.K;
+        const float r = fmaxf(eps, stds[d.cumT + c]);
+        s.x /= r;
+        s.y /= r;
+    }
+    gW[idx] = s;
 }
 
 // --------------------------------------------------------------------------- grad FF
@@ -647,9 +676,13 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     return CGNET_OK;
 }
 
+static int gradw_chunks(int B) { return (B + kGradWChunk - 1) / kGradWChunk; }
+
 extern "C" size_t cgnet_FN_WMM_backward_workspace(const cgnet_wmm_plan* plan, int B) {
     if (!plan || B <= 0) return 0;
-    return align_up(sizeof(float) * 2 * (size_t)plan->nW, 256);
+    // [conj(W)/div, channel-major] [raw weight-gradient sums per chunk of samples]
+    return align_up(sizeof(float) * 2 * (size_t)plan->nW, 256) +
+           align_up(sizeof(float) * 2 * (size_t)plan->nW * gradw_chunks(B), 256);
 }
 
 extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* d_gFF, float* d_gW,
@@ -662,6 +695,11 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
     CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
     hipStream_t s = (hipStream_t)stream;
     const int ndeg = (int)plan->degs.size();
+    const size_t need = cgnet_FN_WMM_backward_workspace(plan, B);
+    CGNET_REQUIRE(B == 0 || (d_workspace && workspace_bytes >= need), CGNET_ERR_WORKSPACE,
+                  "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    float2* WT = (float2*)d_workspace;
+    float2* gw_part = (float2*)((char*)d_workspace + align_up(sizeof(float) * 2 * (size_t)plan->nW, 256));
     if (d_gW && plan->nW > 0) {
         if (B == 0 || plan->nO == 0) {
             const size_t n = (size_t)2 * plan->nW;
@@ -669,9 +707,14 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_HIP(hipGetLastError());
         } else {
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
-            hipLaunchKernelGGL(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size()), dim3(kThreads), 0, s,
-                               (const float2*)d_gO, (const float2*)d_FF, bn ? d_stds : nullptr, eps, (float2*)d_gW,
-                               plan->d_degs, plan->d_gw_units, B, plan->nFF, plan->nO);
+            const int nchunks = gradw_chunks(B);
+            hipLaunchKernelGGL(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), 0, s,
+                               (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
+                               kGradWChunk, plan->nFF, plan->nO, plan->nW);
+            CGNET_HIP(hipGetLastError());
+            hipLaunchKernelGGL(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
+                               (const float2*)gw_part, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg,
+                               (float2*)d_gW, plan->nW, nchunks);
             CGNET_HIP(hipGetLastError());
         }
     }
@@ -679,10 +722,6 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
         CGNET_REQUIRE(d_W, CGNET_ERR_ARG, "d_W is NULL");
         CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
-        const size_t need = cgnet_FN_WMM_backward_workspace(plan, B);
-        CGNET_REQUIRE(d_workspace && workspace_bytes >= need, CGNET_ERR_WORKSPACE,
-                      "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
-        float2* WT = (float2*)d_workspace;
         if (plan->nW > 0) {
             hipLaunchKernelGGL(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
