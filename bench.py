@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one Clebsch-Gordan layer (CG product -> fragment norm -> weight mixing),
+forward + backward, at L=11, tau=12, B=100 (BASELINE.json configs[2]) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Prints ONE JSON line.  A "step" is one training-mode forward (statistics update included) plus
+one backward (input gradient and weight gradient) of the layer over one batch of synthetic
+fragments that already reside in HBM.  `roofline` describes the kernel that takes the most
+time inside the timed region (durations from HIP events the library records on the launch
+stream); `whole_step` prices the complete step against the five compulsory passes over the
+materialised product tensor.  `cpu_baseline` times the CPU oracle (a port of the reference's
+python path) on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published peak
+
+WORKLOAD = {"lmax": 11, "tau": 12, "batch": 100}
+
+
+def synthetic(lmax, tau, bsz, t_ff, seed=0):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = torch.cat([torch.randn(bsz, tau * (2 * l + 1), 2, generator=g) / math.sqrt(2 * l + 1)
+                   for l in range(lmax + 1)], dim=1)
+    w = torch.cat([torch.randn(t_ff[l] * tau, 2, generator=g) / math.sqrt(t_ff[l]) for l in range(lmax + 1)])
+    go = torch.randn(bsz, tau * (lmax + 1) ** 2, 2, generator=g)
+    return x, w, go
+
+
+def cpu_baseline(lmax, tau, codes, t_ff, sample_batch, repeats):
+    """The oracle's float32 layer (port of the reference's python path) on the host cores."""
+    import numpy as np
+    import torch
+    from oracle import cg_layer as OL
+    taus = [tau] * (lmax + 1)
+    x, w, go = synthetic(lmax, tau, sample_batch, t_ff, seed=1)
+    layer = OL.LayerOracle(lmax, taus, taus, codes, batchnorm=True)
+    layer.set_stds_flat(np.ones(sum(t_ff), dtype=np.float32))
+
+    def step():
+        xx = x.clone().requires_grad_(True)
+        ww = w.clone().requires_grad_(True)
+        out = OL.join_straight(layer.forward(xx, ww))
+        out.backward(go)
+        return xx.grad, ww.grad
+    step()                                            # warm-up (also builds the CG matrices)
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        step()
+    dt = (time.perf_counter() - t0) / repeats
+    return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(torch.get_num_threads()),
+            "kind": "port",
+            "sample": "B=%d of the same L=%d tau=%d layer fwd+bwd, float32 torch CPU oracle, 1 warm-up + %d timed "
+                      "steps, %.1f s per step" % (sample_batch, lmax, tau, repeats, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--cpu-repeats", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build runs the CG layer on ONE GPU (no collectives, no sharding); "
+                         "--gpus %d is not supported.\n" % args.gpus)
+        sys.exit(2)
+
+    import torch
+    from cgnet_amd import CG_layers, _lib
+    lib = _lib.load()
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    lmax, tau, bsz = WORKLOAD["lmax"], WORKLOAD["tau"], WORKLOAD["batch"]
+    taus = [tau] * (lmax + 1)
+    layer = CG_layers.CGBN_cuda(lmax, taus, taus, batchnorm=True, sparse_flag=False, device=dev)
+    t_ff = [int(v) for v in layer.t_FF]
+    x, w, go = synthetic(lmax, tau, bsz, t_ff)
+    with torch.no_grad():
+        layer.bnWMM.W.copy_(w)
+        layer.bnWMM.bn_stds.fill_(1.0)
+    x = x.to(dev).requires_grad_(True)
+    go = go.to(dev)
+    layer.train()
+
+    def step():
+        x.grad = None
+        layer.bnWMM.W.grad = None
+        out = layer(x, straight_output=True)
+        out.backward(go)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.cgnet_profile_reset()
+    lib.cgnet_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.cgnet_profile_enable(0)
+    times = _lib.kernel_times()
+    assert torch.isfinite(x.grad).all() and torch.isfinite(layer.bnWMM.W.grad).all()
+
+    n_f = tau * (lmax + 1) ** 2
+    n_o = n_f
+    n_ff = int(layer.cg.cumu_tm_FF[-1])
+    n_w = int(layer.bnWMM.W.shape[0])
+    sum_t = sum(t_ff)
+    cg_len = int(layer.cg.CGspace.numel())
+    # algorithmic bytes per launch of the five kernels that stream the product tensor
+    algo = {
+        "cg_forward_kernel": 8 * bsz * (n_f + n_ff),
+        "wmm_forward_kernel": 8 * (bsz * n_ff + n_w + bsz * n_o) + 4 * sum_t,
+        "wmm_gradw_kernel": 8 * (bsz * n_ff + bsz * n_o + n_w),
+        "wmm_gradff_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
+        "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
+    }
+    step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
+    kernels = {}
+    for name, (ms, cnt) in sorted(times.items(), key=lambda kv: -kv[1][0]):
+        avg = ms / max(cnt, 1)
+        ent = {"avg_ms": round(avg, 4), "launches_per_step": cnt / args.steps}
+        if name in algo and avg > 0:
+            ent["algorithmic_GBps"] = round(algo[name] / (avg * 1e-3) / 1e9, 1)
+        kernels[name] = ent
+    dominant = max((n for n in times if n in algo), key=lambda n: times[n][0])
+    d_avg_s = times[dominant][0] / times[dominant][1] * 1e-3
+    achieved = algo[dominant] / d_avg_s / 1e9
+    ms_per_step = dt / args.steps * 1e3
+
+    line = {
+        "metric": "CG-layer fwd+bwd samples/sec at L=11,tau=12,B=100; % HBM roofline",
+        "value": bsz * args.steps / dt,
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[2]: one CGNet layer fwd+bwd, Lmax=11, tau=12, B=100, fp32 complex, "
+                               "CG product + fragment norm + weight mixing, default (l2<=l1) triples",
+                   "lmax": lmax, "tau": tau, "batch": bsz, "triples": len(layer.cg.lll_list)},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": algo[dominant], "avg_launch_ms": d_avg_s * 1e3},
+        "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
+                       "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        del x, go
+        torch.cuda.empty_cache()
+        line["cpu_baseline"] = cpu_baseline(lmax, tau, layer.cg.lll_list, t_ff, args.cpu_batch, args.cpu_repeats)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -40,6 +40,11 @@ SIGNATURES = {
     "cgnet_FN_WMM_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_FN_WMM_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                              ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_profile_enable": (ctypes.c_int, [ctypes.c_int]),
+    "cgnet_profile_reset": (ctypes.c_int, []),
+    "cgnet_profile_collect": (ctypes.c_int, []),
+    "cgnet_profile_get": (ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, ctypes.c_int,
+                                         ctypes.POINTER(ctypes.c_double), _c_int_p]),
 }
 
 _lib = None
@@ -76,3 +81,17 @@ def check(code):
 def int_array(values):
     values = [int(v) for v in values]
     return (ctypes.c_int * max(1, len(values)))(*values)
+
+
+def kernel_times():
+    """{kernel name: (total milliseconds, launches)} gathered since the last reset.
+    The caller must have synchronised the device first."""
+    lib = load()
+    n = lib.cgnet_profile_collect()
+    out = {}
+    buf = ctypes.create_string_buffer(128)
+    for i in range(n):
+        ms, cnt = ctypes.c_double(), ctypes.c_int()
+        check(lib.cgnet_profile_get(i, buf, len(buf), ctypes.byref(ms), ctypes.byref(cnt)))
+        out[buf.value.decode()] = (ms.value, cnt.value)
+    return out

@@ -587,7 +587,7 @@ static int launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF,
     if (ntasks == 0 || B == 0) return CGNET_OK;
     const int ngroups = (B + spg - 1) / spg;
     CGNET_REQUIRE(ngroups <= 65535, CGNET_ERR_UNSUPPORTED, "batch of %d needs %d sample groups (limit 65535)", B, ngroups);
-    hipLaunchKernelGGL(cg_forward_kernel, dim3(ntasks, ngroups), dim3(kThreads), p->fwd_lds, s,
+    CGNET_LAUNCH(cg_forward_kernel, dim3(ntasks, ngroups), dim3(kThreads), p->fwd_lds, s,
                        (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks, p->nF, p->nFF, B, spg, d_part, p->sumT);
     CGNET_HIP(hipGetLastError());
     return CGNET_OK;
@@ -633,7 +633,7 @@ extern "C" int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float
     int rc = launch_forward(plan, d_F, d_FF, d_CG, B, (double*)d_workspace, spg, s);
     if (rc != CGNET_OK) return rc;
     const int n2 = 2 * plan->sumT;
-    hipLaunchKernelGGL(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
+    CGNET_LAUNCH(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
                        (const double*)d_workspace, d_sums, n2, ngroups);
     CGNET_HIP(hipGetLastError());
     return CGNET_OK;
@@ -668,13 +668,13 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
                   "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     const int* d_gb = plan->d_bwd_group_table + plan->bwd_group_table_off[ng];
     float2* dst = ng > 1 ? (float2*)d_workspace : (float2*)d_gF;
-    hipLaunchKernelGGL(cg_backward_kernel, dim3(ng, B), dim3(kThreads), plan->bwd_lds, s,
+    CGNET_LAUNCH(cg_backward_kernel, dim3(ng, B), dim3(kThreads), plan->bwd_lds, s,
                        (const float2*)d_F, (const float2*)d_gFF, d_CG, dst, plan->d_bwd_tasks, d_gb,
                        plan->nF, plan->nFF, B, 0);
     CGNET_HIP(hipGetLastError());
     if (ng > 1) {
         const size_t n = (size_t)plan->nF * B;
-        hipLaunchKernelGGL(partial_sum_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+        CGNET_LAUNCH(partial_sum_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
                            (const float2*)d_workspace, (float2*)d_gF, n, ng);
         CGNET_HIP(hipGetLastError());
     }

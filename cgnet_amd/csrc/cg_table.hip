@@ -74,7 +74,7 @@ extern "C" int cgnet_sparse_precomputeCG(float* d_CG, int L, const int* h_llls, 
     CGNET_HIP(hipMallocAsync((void**)&d_tr, sizeof(TableTriple) * nllls, s));
     CGNET_HIP(hipMemcpyAsync(d_tr, tr.data(), sizeof(TableTriple) * nllls, hipMemcpyHostToDevice, s));
     const int nfact = 3 * L + 2;   // largest argument is l1 + l2 + l + 1
-    hipLaunchKernelGGL(cg_table_kernel, dim3(nllls), dim3(256), sizeof(double) * nfact, s, d_CG, d_tr, nfact);
+    CGNET_LAUNCH(cg_table_kernel, dim3(nllls), dim3(256), sizeof(double) * nfact, s, d_CG, d_tr, nfact);
     CGNET_HIP(hipGetLastError());
     // the host vector must outlive the async copy
     CGNET_HIP(hipStreamSynchronize(s));

@@ -35,4 +35,22 @@ constexpr int kMaxTau = 1024;      // channels of one degree
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Optional per-kernel timing (cgnet_profile_*): when enabled, every launch is bracketed by a
+// pair of HIP events recorded on the launch stream.
+class KernelTimer {
+public:
+    KernelTimer(const char* name, hipStream_t stream);
+    ~KernelTimer();
+private:
+    const char* name_;
+    hipStream_t stream_;
+    hipEvent_t start_ = nullptr, stop_ = nullptr;
+};
+
+#define CGNET_LAUNCH(kernel, grid, block, lds, stream, ...)                                   \
+    do {                                                                                      \
+        ::cgnet::KernelTimer timer__(#kernel, stream);                                        \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                    \
+    } while (0)
+
 }  // namespace cgnet

@@ -623,30 +623,30 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
             const int ng = stat_groups_for(B);
             const int spg = (B + ng - 1) / ng;
             const int ngroups = (B + spg - 1) / spg;
-            hipLaunchKernelGGL(fn_stats_kernel, dim3((unsigned)plan->stat_units.size(), ngroups), dim3(kThreads),
+            CGNET_LAUNCH(fn_stats_kernel, dim3((unsigned)plan->stat_units.size(), ngroups), dim3(kThreads),
                                plan->stat_lds, s, (const float2*)d_FF, plan->d_degs, plan->d_stat_units, plan->nFF,
                                B, spg, (double*)(base + ws.part), plan->sumT);
             CGNET_HIP(hipGetLastError());
             const int n2 = 2 * plan->sumT;
-            hipLaunchKernelGGL(fn_sum_groups_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
+            CGNET_LAUNCH(fn_sum_groups_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
                                (const double*)(base + ws.part), (double*)(base + ws.sums), n2, ngroups);
             CGNET_HIP(hipGetLastError());
             sums = (const double*)(base + ws.sums);
         }
-        hipLaunchKernelGGL(fn_update_std_kernel, dim3((plan->sumT + 255) / 256), dim3(256), 0, s, sums, d_stds,
+        CGNET_LAUNCH(fn_update_std_kernel, dim3((plan->sumT + 255) / 256), dim3(256), 0, s, sums, d_stds,
                            plan->d_degs, ndeg, plan->sumT, B, cnt);
         CGNET_HIP(hipGetLastError());
     }
     if (plan->nO == 0) return CGNET_OK;
     if (plan->fwd_units.empty()) {   // degrees with outputs but no mid channels produce zeros
         const size_t n = (size_t)2 * plan->nO * B;
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_O, n);
+        CGNET_LAUNCH(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_O, n);
         CGNET_HIP(hipGetLastError());
         return CGNET_OK;
     }
     float* Wp = (float*)(base + ws.wp);
     const int total = plan->wp_blocks * 64;
-    hipLaunchKernelGGL(pack_w_forward_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
+    CGNET_LAUNCH(pack_w_forward_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
                        bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Wp, plan->wp_blocks);
     CGNET_HIP(hipGetLastError());
     // degrees with t_O > 0 but no mid channels are never written by the product kernel
@@ -656,7 +656,7 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     if (holes || plan->maxS > 1) {
         const size_t n = (size_t)2 * plan->nO * B * (plan->maxS > 1 ? plan->maxS : 1);
         if (holes) {
-            hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)out, n);
+            CGNET_LAUNCH(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)out, n);
             CGNET_HIP(hipGetLastError());
         }
     }
@@ -664,12 +664,12 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     for (const WmmDeg& d : plan->degs)
         if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + d.G - 1) / d.G);
     CGNET_REQUIRE(ygroups <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d too large", B);
-    hipLaunchKernelGGL(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads), 0, s,
+    CGNET_LAUNCH(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads), 0, s,
                        d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO);
     CGNET_HIP(hipGetLastError());
     if (plan->maxS > 1) {
         const size_t n = (size_t)plan->nO * B;
-        hipLaunchKernelGGL(wmm_sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+        CGNET_LAUNCH(wmm_sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
                            (const float2*)out, (float2*)d_O, plan->d_cumO, ndeg, B, plan->nO);
         CGNET_HIP(hipGetLastError());
     }
@@ -703,16 +703,16 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
     if (d_gW && plan->nW > 0) {
         if (B == 0 || plan->nO == 0) {
             const size_t n = (size_t)2 * plan->nW;
-            hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gW, n);
+            CGNET_LAUNCH(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gW, n);
             CGNET_HIP(hipGetLastError());
         } else {
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
             const int nchunks = gradw_chunks(B);
-            hipLaunchKernelGGL(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), 0, s,
+            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), 0, s,
                                (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
                                kGradWChunk, plan->nFF, plan->nO, plan->nW);
             CGNET_HIP(hipGetLastError());
-            hipLaunchKernelGGL(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
+            CGNET_LAUNCH(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)gw_part, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg,
                                (float2*)d_gW, plan->nW, nchunks);
             CGNET_HIP(hipGetLastError());
@@ -723,11 +723,11 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         CGNET_REQUIRE(d_W, CGNET_ERR_ARG, "d_W is NULL");
         CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
         if (plan->nW > 0) {
-            hipLaunchKernelGGL(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
+            CGNET_LAUNCH(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
             CGNET_HIP(hipGetLastError());
         }
-        hipLaunchKernelGGL(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
+        CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
                            plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
                            plan->d_gff_units, plan->nFF, plan->nO);
         CGNET_HIP(hipGetLastError());

@@ -138,6 +138,18 @@ int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* 
                           float eps, int flags,
                           void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* ---- measurement hooks (no counterpart in the reference, which times nothing) ------------ */
+
+/* With timing enabled every kernel launch of this library is bracketed by two HIP events
+ * recorded on the launch stream.  After the caller has synchronised those streams,
+ * cgnet_profile_collect() folds the finished pairs into per-kernel totals and returns the
+ * number of distinct kernels; cgnet_profile_get(i, ...) reads entry i (name, summed
+ * milliseconds, launches).  cgnet_profile_enable returns the previous setting. */
+int cgnet_profile_enable(int on);
+int cgnet_profile_reset(void);
+int cgnet_profile_collect(void);
+int cgnet_profile_get(int index, char* name, int name_capacity, double* total_ms, int* launches);
+
 #ifdef __cplusplus
 }
 #endif
