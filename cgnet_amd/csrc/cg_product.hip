@@ -16,6 +16,8 @@
 // and combines with a fixed DPP tree, so the result does not depend on scheduling.  Groups
 // write partial gradients that a second kernel adds in a fixed order.
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <memory>
 #include <vector>
 
@@ -33,6 +35,27 @@ struct CgTask {
     int cg_off;           // float offset of the triple's table
     int chan0;            // index over all mid channels (all degrees) of the tile's first channel
     int nT1, nT2, TI, TJ; // forward register tiling: rows = nT1 x TI (strided), tau2 = nT2 x TJ
+    int bTI[2], bRW[2];   // backward, per slot: output channels per thread, lanes sharing one output
+};
+
+// Backward, register-resident scheme: one work-group per (sample, unit), a unit being the
+// triples that share l1 restricted to a range of t1 rows.
+struct BwdUnit {
+    int l1, rows;
+    int offF1;                // complex offset inside a sample's F of the unit's first row
+    int task_begin, task_end; // range in the unit-ordered task array (sorted by l2, then l)
+    int nA;                   // waves that take slot 1; the other waves of the group take slot 2
+    int TI, RW;               // slot-1 tiling: output rows per thread, lanes sharing one output
+};
+
+struct BwdUTask {
+    int l, l2, tau2;
+    int offFF;                // complex offset inside a sample's gFF of the tile
+    int offF2;                // complex offset inside a sample's F of degree l2
+    int cg_off;
+    int p2off;                // complex offset inside a sample's slot-2 partial area of this (unit, l2) slab
+    int first_of_l2, last_of_l2;
+    int TI, RW;               // slot-2 tiling for this run of equal l2
 };
 
 }  // namespace cgnet
@@ -48,6 +71,16 @@ struct cgnet_cg_plan {
     std::vector<int> bwd_group_table_off;        // for ng groups: first entry of its ng+1 boundaries
     int* d_bwd_group_table = nullptr;
     size_t fwd_lds = 0, bwd_lds = 0;
+    int bwd_threads = 256;                       // work-group size of the backward kernel
+    // register-resident backward (used when every unit fits; otherwise the LDS-accumulator kernel)
+    bool bwd_fast = false;
+    std::vector<cgnet::BwdUnit> bwd_units;
+    std::vector<cgnet::BwdUTask> bwd_utasks;
+    cgnet::BwdUnit* d_bwd_units = nullptr;
+    cgnet::BwdUTask* d_bwd_utasks = nullptr;
+    int* d_bwd_combine = nullptr;                // [L+2] cumF | [L+1] own1 | [L+2] list begin | list of slab offsets
+    int bwd_P2 = 0;                              // complex entries of one sample's slot-2 partial area
+    size_t bwd_fast_lds = 0;
     int device = 0;
 };
 
@@ -226,135 +259,596 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
-constexpr int kBT = 4;   // output rows per thread in the backward phases
+// Zero padding of the m axis of the staged gFF tile and of the CG table rows: the two m
+// outputs of a thread and the two-step unrolled loop may touch one index below and two above.
+constexpr int kPadLo = 1, kPadHi = 2;
+
+__host__ __device__ inline size_t bwd_task_lds(const CgTask& t) {
+    const size_t M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
+    const size_t Mp = M + kPadLo + kPadHi;
+    return 8 * ((size_t)t.rows * t.tau2 * Mp + (size_t)t.rows * M1 + (size_t)t.tau2 * M2) + 4 * Mp * M2;
+}
 
 // Gradient with respect to the slot that is NOT reduced over.
 //   SLOT == 1: outputs (t1 in the task's rows, m1), reduced over (t2, m2)
 //   SLOT == 2: outputs (t2, m2),                    reduced over (t1 in rows, m1)
-// g is the staged gFF tile [rows][tau2][M]; fr the staged fragments of the reduced slot;
-// acc the sample-wide gradient accumulator; out_base the complex offset of the output slab.
-template <int SLOT, int RW>
-__device__ __forceinline__ void bwd_phase(const CgTask& t, const float* __restrict__ cg,
+// A thread owns TI output channels x 2 consecutive m; RW lanes share one such item and split
+// the reduced channels, then add up over a fixed DPP tree.  Along the reduced m the two
+// outputs read a sliding two-element window of the staged gFF tile (g, rows padded with zeros),
+// so a step costs TI + 1 + 2 LDS reads for 2*TI complex multiply-adds.
+template <int SLOT, int TI, int RW>
+__device__ __forceinline__ void bwd_phase(const CgTask& t, const float* __restrict__ cgp,
                                           const float2* __restrict__ g, const float2* __restrict__ fr,
-                                          float2* __restrict__ acc) {
+                                          float2* __restrict__ acc, int nthreads) {
     const int l = t.l, l1 = t.l1, l2 = t.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
+    const int Mp = M + kPadLo + kPadHi;
     const int rows = t.rows, tau2 = t.tau2;
-    // geometry of the output slot (o) and the reduced slot (r)
     const int n_o = (SLOT == 1) ? rows : tau2;        // output channels
     const int n_r = (SLOT == 1) ? tau2 : rows;        // reduced channels
-    const int l_o = (SLOT == 1) ? l1 : l2, l_r = (SLOT == 1) ? l2 : l1;
     const int M_o = (SLOT == 1) ? M1 : M2, M_r = (SLOT == 1) ? M2 : M1;
-    const int g_so = (SLOT == 1) ? tau2 * M : M;      // stride in g between output channels
-    const int g_sr = (SLOT == 1) ? M : tau2 * M;      // stride in g between reduced channels
+    const int g_so = (SLOT == 1) ? tau2 * Mp : Mp;    // stride in g between output channels
+    const int g_sr = (SLOT == 1) ? Mp : tau2 * Mp;    // stride in g between reduced channels
     const int out_base = (SLOT == 1) ? t.offF1 : t.offF2;
+    const int d = l1 + l2 - l;                        // m index of g = mo + mr - d (all 0-based)
 
-    constexpr int nrows_blk = kThreads / RW;
+    const int nrows_blk = nthreads / RW;
     const int row_id = threadIdx.x / RW, lane_r = threadIdx.x % RW;
-    const int nT = (n_o + kBT - 1) / kBT;
-    const int nitems = nT * M_o;
+    const int nT = (n_o + TI - 1) / TI;
+    const int nWin = (M_o + 1) >> 1;
+    const int nitems = nT * nWin;
     const int npass = (nitems + nrows_blk - 1) / nrows_blk;
     for (int pass = 0; pass < npass; ++pass) {
         const int item = pass * nrows_blk + row_id;
         const bool valid = item < nitems;
-        float ax[kBT], ay[kBT];
+        float ax[TI][2], ay[TI][2];
 #pragma unroll
-        for (int i = 0; i < kBT; ++i) ax[i] = ay[i] = 0.f;
-        int mmo = 0, to = 0;
+        for (int i = 0; i < TI; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+        int mo0 = 0, to = 0;
         if (valid) {
-            mmo = item % M_o;
-            to = item / M_o;
-            const int mo = mmo - l_o;
-            const int lo = max(-l_r, -l - mo), hi = min(l_r, l - mo);
-            int go[kBT];
+            const int w = item % nWin;
+            to = item / nWin;
+            mo0 = 2 * w;
+            // reduced-m range in which at least one of the two outputs has 0 <= m index < M
+            const int ir_lo = max(0, d - mo0 - 1);
+            const int ir_hi = min(M_r - 1, M - 1 + d - mo0);
+            int go[TI];
 #pragma unroll
-            for (int i = 0; i < kBT; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
+            for (int i = 0; i < TI; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
+            const int col0 = min(mo0, M2 - 1), col1 = min(mo0 + 1, M2 - 1);   // SLOT 2: table columns
             for (int r = lane_r; r < n_r; r += RW) {
-                const float2* frow = fr + r * M_r + l_r;
-                const float2* grow = g + r * g_sr + (mo + l);
-                for (int mr = lo; mr <= hi; ++mr) {
-                    // table entry [m + l][m2 + l2] with m = mo + mr
-                    const float c = (SLOT == 1) ? cg[(mo + mr + l) * M2 + (mr + l2)]
-                                                : cg[(mo + mr + l) * M2 + mmo];
-                    const float2 f = frow[mr];
-                    const float cx = c * f.x, cy = -c * f.y;   // c * conj(f)
+                const float2* frow = fr + r * M_r;
+                const float2* gb = g + r * g_sr + (kPadLo + mo0 - d);          // gb[ch + ir] = g[.., m = mo0+ir-d]
+                const float* cb = cgp + (kPadLo + mo0 - d) * M2;               // cb[ir*M2 + col] = table row mo0+ir-d
+                float2 e0[TI], e1[TI];
 #pragma unroll
-                    for (int i = 0; i < kBT; ++i) {
-                        const float2 gv = grow[go[i] + mr];
-                        ax[i] = fmaf(gv.x, cx, ax[i]);
-                        ax[i] = fmaf(-gv.y, cy, ax[i]);
-                        ay[i] = fmaf(gv.x, cy, ay[i]);
-                        ay[i] = fmaf(gv.y, cx, ay[i]);
+                for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir_lo];
+                for (int ir = ir_lo; ir <= ir_hi; ir += 2) {
+                    // ---- step ir: outputs (mo0, mo0+1) read (e0, e1)
+#pragma unroll
+                    for (int i = 0; i < TI; ++i) e1[i] = gb[go[i] + ir + 1];
+                    {
+                        const float2 f = frow[ir];
+                        const float c0 = (SLOT == 1) ? cb[ir * M2 + ir] : cb[ir * M2 + col0];
+                        const float c1 = (SLOT == 1) ? cb[(ir + 1) * M2 + ir] : cb[(ir + 1) * M2 + col1];
+                        const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
+#pragma unroll
+                        for (int i = 0; i < TI; ++i) {
+                            ax[i][0] = fmaf(e0[i].x, c0x, ax[i][0]);
+                            ax[i][0] = fmaf(-e0[i].y, c0y, ax[i][0]);
+                            ay[i][0] = fmaf(e0[i].x, c0y, ay[i][0]);
+                            ay[i][0] = fmaf(e0[i].y, c0x, ay[i][0]);
+                            ax[i][1] = fmaf(e1[i].x, c1x, ax[i][1]);
+                            ax[i][1] = fmaf(-e1[i].y, c1y, ax[i][1]);
+                            ay[i][1] = fmaf(e1[i].x, c1y, ay[i][1]);
+                            ay[i][1] = fmaf(e1[i].y, c1x, ay[i][1]);
+                        }
+                    }
+                    // ---- step ir+1: the window has moved by one, roles of e0 / e1 swap
+#pragma unroll
+                    for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir + 2];
+                    {
+                        const int ir1 = ir + 1;
+                        const int irc = min(ir1, M_r - 1);
+                        float2 f = frow[irc];
+                        if (ir1 > ir_hi) f = make_float2(0.f, 0.f);
+                        const float c0 = (SLOT == 1) ? cb[ir1 * M2 + irc] : cb[ir1 * M2 + col0];
+                        const float c1 = (SLOT == 1) ? cb[(ir1 + 1) * M2 + irc] : cb[(ir1 + 1) * M2 + col1];
+                        const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
+#pragma unroll
+                        for (int i = 0; i < TI; ++i) {
+                            ax[i][0] = fmaf(e1[i].x, c0x, ax[i][0]);
+                            ax[i][0] = fmaf(-e1[i].y, c0y, ax[i][0]);
+                            ay[i][0] = fmaf(e1[i].x, c0y, ay[i][0]);
+                            ay[i][0] = fmaf(e1[i].y, c0x, ay[i][0]);
+                            ax[i][1] = fmaf(e0[i].x, c1x, ax[i][1]);
+                            ax[i][1] = fmaf(-e0[i].y, c1y, ax[i][1]);
+                            ay[i][1] = fmaf(e0[i].x, c1y, ay[i][1]);
+                            ay[i][1] = fmaf(e0[i].y, c1x, ay[i][1]);
+                        }
                     }
                 }
             }
         }
 #pragma unroll
-        for (int i = 0; i < kBT; ++i) {
-            ax[i] = row_sum<RW>(ax[i]);
-            ay[i] = row_sum<RW>(ay[i]);
+        for (int i = 0; i < TI; ++i) {
+            ax[i][0] = row_sum<RW>(ax[i][0]);
+            ay[i][0] = row_sum<RW>(ay[i][0]);
+            ax[i][1] = row_sum<RW>(ax[i][1]);
+            ay[i][1] = row_sum<RW>(ay[i][1]);
         }
-        if (valid && lane_r == 0) {
+        if (valid) {
 #pragma unroll
-            for (int i = 0; i < kBT; ++i) {
-                const int ch = to + nT * i;
-                if (ch < n_o) {
-                    float2* p = acc + out_base + ch * M_o + mmo;
-                    float2 v = *p;
-                    v.x += ax[i];
-                    v.y += ay[i];
-                    *p = v;
+            for (int k = 0; k < 2; ++k) {
+                if (lane_r != (k % RW)) continue;        // lane k of the row stores output k
+                const int mo = mo0 + k;
+                if (mo >= M_o) continue;
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    const int ch = to + nT * i;
+                    if (ch < n_o) {
+                        float2* p = acc + out_base + ch * M_o + mo;
+                        float2 v = *p;
+                        v.x += ax[i][k];
+                        v.y += ay[i][k];
+                        *p = v;
+                    }
                 }
             }
         }
     }
 }
 
+template <int SLOT, int TI>
+__device__ __forceinline__ void bwd_phase_rw(int rw, const CgTask& t, const float* cgp, const float2* g,
+                                             const float2* fr, float2* acc, int nthreads) {
+    switch (rw) {
+        case 1: bwd_phase<SLOT, TI, 1>(t, cgp, g, fr, acc, nthreads); break;
+        case 2: bwd_phase<SLOT, TI, 2>(t, cgp, g, fr, acc, nthreads); break;
+        case 4: bwd_phase<SLOT, TI, 4>(t, cgp, g, fr, acc, nthreads); break;
+        case 8: bwd_phase<SLOT, TI, 8>(t, cgp, g, fr, acc, nthreads); break;
+        default: bwd_phase<SLOT, TI, 16>(t, cgp, g, fr, acc, nthreads); break;
+    }
+}
+
 template <int SLOT>
-__device__ __forceinline__ void bwd_phase_dispatch(int n_reduce, const CgTask& t, const float* cg,
-                                                   const float2* g, const float2* fr, float2* acc) {
-    if (n_reduce <= 1) bwd_phase<SLOT, 1>(t, cg, g, fr, acc);
-    else if (n_reduce <= 2) bwd_phase<SLOT, 2>(t, cg, g, fr, acc);
-    else if (n_reduce <= 4) bwd_phase<SLOT, 4>(t, cg, g, fr, acc);
-    else if (n_reduce <= 8) bwd_phase<SLOT, 8>(t, cg, g, fr, acc);
-    else bwd_phase<SLOT, 16>(t, cg, g, fr, acc);
+__device__ __forceinline__ void bwd_phase_dispatch(const CgTask& t, const float* cgp, const float2* g,
+                                                   const float2* fr, float2* acc, int nthreads) {
+    const int ti = t.bTI[SLOT - 1], rw = t.bRW[SLOT - 1];
+    switch (ti) {
+        case 1: bwd_phase_rw<SLOT, 1>(rw, t, cgp, g, fr, acc, nthreads); break;
+        case 2: bwd_phase_rw<SLOT, 2>(rw, t, cgp, g, fr, acc, nthreads); break;
+        case 3: bwd_phase_rw<SLOT, 3>(rw, t, cgp, g, fr, acc, nthreads); break;
+        default: bwd_phase_rw<SLOT, 4>(rw, t, cgp, g, fr, acc, nthreads); break;
+    }
 }
 
 __global__ void __launch_bounds__(kThreads)
 cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
                    const float* __restrict__ CG, float2* __restrict__ dst,
                    const CgTask* __restrict__ tasks, const int* __restrict__ group_begin,
-                   int nF, int nFF, int B, int tile_floats2) {
+                   int nF, int nFF, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
     float2* acc = reinterpret_cast<float2*>(smem);
     float2* g = acc + nF;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, nthreads = blockDim.x;
     const int b = blockIdx.y, grp = blockIdx.x;
-    for (int e = tid; e < nF; e += kThreads) acc[e] = make_float2(0.f, 0.f);
+    for (int e = tid; e < nF; e += nthreads) acc[e] = make_float2(0.f, 0.f);
     const float2* Fb = F + (size_t)b * nF;
     const float2* Gb = gFF + (size_t)b * nFF;
     const int tbeg = group_begin[grp], tend = group_begin[grp + 1];
     for (int ti = tbeg; ti < tend; ++ti) {
         const CgTask t = tasks[ti];
         const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
-        const int nout = t.rows * t.tau2 * M, n1 = t.rows * M1, n2 = t.tau2 * M2, ncg = M * M2;
-        float2* f1 = g + nout;
+        const int Mp = M + kPadLo + kPadHi;
+        const int nch = t.rows * t.tau2;
+        const int n1 = t.rows * M1, n2 = t.tau2 * M2;
+        float2* f1 = g + nch * Mp;
         float2* f2 = f1 + n1;
-        float* cg = reinterpret_cast<float*>(f2 + n2);
+        float* cgp = reinterpret_cast<float*>(f2 + n2);
         __syncthreads();   // previous task (and the zeroing) done before the staging area is reused
-        for (int e = tid; e < nout; e += kThreads) g[e] = Gb[t.offFF + e];
-        for (int e = tid; e < n1; e += kThreads) f1[e] = Fb[t.offF1 + e];
-        for (int e = tid; e < n2; e += kThreads) f2[e] = Fb[t.offF2 + e];
-        for (int e = tid; e < ncg; e += kThreads) cg[e] = CG[t.cg_off + e];
+        {
+            const float inv = 1.0f / (float)Mp;
+            const float2* src = Gb + t.offFF;
+            for (int e = tid; e < nch * Mp; e += nthreads) {
+                const int ch = (int)(((float)e + 0.5f) * inv);
+                const int x = e - ch * Mp - kPadLo;
+                float2 v = make_float2(0.f, 0.f);
+                if (x >= 0 && x < M) v = src[ch * M + x];
+                g[e] = v;
+            }
+        }
+        for (int e = tid; e < n1; e += nthreads) f1[e] = Fb[t.offF1 + e];
+        for (int e = tid; e < n2; e += nthreads) f2[e] = Fb[t.offF2 + e];
+        for (int e = tid; e < Mp * M2; e += nthreads) {
+            const int x = e - kPadLo * M2;
+            cgp[e] = (x >= 0 && x < M * M2) ? CG[t.cg_off + x] : 0.f;
+        }
         __syncthreads();
-        bwd_phase_dispatch<1>(t.tau2, t, cg, g, f2, acc);
+        bwd_phase_dispatch<1>(t, cgp, g, f2, acc, nthreads);
         __syncthreads();   // a diagonal triple writes the same slab in both phases
-        bwd_phase_dispatch<2>(t.rows, t, cg, g, f1, acc);
+        bwd_phase_dispatch<2>(t, cgp, g, f1, acc, nthreads);
     }
     __syncthreads();
     float2* out = dst + ((size_t)grp * B + b) * nF;
-    for (int e = tid; e < nF; e += kThreads) out[e] = acc[e];
-    (void)tile_floats2;
+    for (int e = tid; e < nF; e += nthreads) out[e] = acc[e];
+}
+
+// ---- register-resident backward ------------------------------------------------------------
+struct BwdGeom { int l, l1, l2, rows, tau2; };
+
+// Adds one task's contribution to the calling thread's accumulators.  Same arithmetic and item
+// layout as bwd_phase, one item per thread (rtid = thread index inside its role), no reduction.
+template <int SLOT, int TI, int RW>
+__device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restrict__ cgp,
+                                          const float2* __restrict__ g, const float2* __restrict__ fr,
+                                          int rtid, float (&ax)[4][2], float (&ay)[4][2]) {
+    const int l = q.l, l1 = q.l1, l2 = q.l2;
+    const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
+    const int Mp = M + kPadLo + kPadHi;
+    const int rows = q.rows, tau2 = q.tau2;
+    const int n_o = (SLOT == 1) ? rows : tau2;
+    const int n_r = (SLOT == 1) ? tau2 : rows;
+    const int M_o = (SLOT == 1) ? M1 : M2, M_r = (SLOT == 1) ? M2 : M1;
+    const int g_so = (SLOT == 1) ? tau2 * Mp : Mp;
+    const int g_sr = (SLOT == 1) ? Mp : tau2 * Mp;
+    const int d = l1 + l2 - l;
+    const int item = rtid / RW, lane_r = rtid % RW;
+    const int nT = (n_o + TI - 1) / TI;
+    const int nWin = (M_o + 1) >> 1;
+    if (item >= nT * nWin) return;
+    const int w = item % nWin, to = item / nWin;
+    const int mo0 = 2 * w;
+    const int ir_lo = max(0, d - mo0 - 1);
+    const int ir_hi = min(M_r - 1, M - 1 + d - mo0);
+    int go[TI];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
+    const int col0 = min(mo0, M2 - 1), col1 = min(mo0 + 1, M2 - 1);
+    for (int r = lane_r; r < n_r; r += RW) {
+        const float2* frow = fr + r * M_r;
+        const float2* gb = g + r * g_sr + (kPadLo + mo0 - d);
+        const float* cb = cgp + (kPadLo + mo0 - d) * M2;
+        float2 e0[TI], e1[TI];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir_lo];
+        for (int ir = ir_lo; ir <= ir_hi; ir += 2) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i) e1[i] = gb[go[i] + ir + 1];
+            {
+                const float2 f = frow[ir];
+                const float c0 = (SLOT == 1) ? cb[ir * M2 + ir] : cb[ir * M2 + col0];
+                const float c1 = (SLOT == 1) ? cb[(ir + 1) * M2 + ir] : cb[(ir + 1) * M2 + col1];
+                const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    ax[i][0] = fmaf(e0[i].x, c0x, ax[i][0]);
+                    ax[i][0] = fmaf(-e0[i].y, c0y, ax[i][0]);
+                    ay[i][0] = fmaf(e0[i].x, c0y, ay[i][0]);
+                    ay[i][0] = fmaf(e0[i].y, c0x, ay[i][0]);
+                    ax[i][1] = fmaf(e1[i].x, c1x, ax[i][1]);
+                    ax[i][1] = fmaf(-e1[i].y, c1y, ax[i][1]);
+                    ay[i][1] = fmaf(e1[i].x, c1y, ay[i][1]);
+                    ay[i][1] = fmaf(e1[i].y, c1x, ay[i][1]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir + 2];
+            {
+                const int ir1 = ir + 1;
+                const int irc = min(ir1, M_r - 1);
+                float2 f = frow[irc];
+                if (ir1 > ir_hi) f = make_float2(0.f, 0.f);
+                const float c0 = (SLOT == 1) ? cb[ir1 * M2 + irc] : cb[ir1 * M2 + col0];
+                const float c1 = (SLOT == 1) ? cb[(ir1 + 1) * M2 + irc] : cb[(ir1 + 1) * M2 + col1];
+                const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    ax[i][0] = fmaf(e1[i].x, c0x, ax[i][0]);
+                    ax[i][0] = fmaf(-e1[i].y, c0y, ax[i][0]);
+                    ay[i][0] = fmaf(e1[i].x, c0y, ay[i][0]);
+                    ay[i][0] = fmaf(e1[i].y, c0x, ay[i][0]);
+                    ax[i][1] = fmaf(e0[i].x, c1x, ax[i][1]);
+                    ax[i][1] = fmaf(-e0[i].y, c1y, ax[i][1]);
+                    ay[i][1] = fmaf(e0[i].x, c1y, ay[i][1]);
+                    ay[i][1] = fmaf(e0[i].y, c1x, ay[i][1]);
+                }
+            }
+        }
+    }
+}
+
+// Adds up the RW lanes of every item (all lanes of the wave take part) and stores the slab
+// dst[n_o][M_o]; every element of the slab has exactly one owner.  Clears the accumulators.
+template <int TI, int RW>
+__device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax)[4][2], float (&ay)[4][2],
+                                          float2* __restrict__ dst) {
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        ax[i][0] = row_sum<RW>(ax[i][0]);
+        ay[i][0] = row_sum<RW>(ay[i][0]);
+        ax[i][1] = row_sum<RW>(ax[i][1]);
+        ay[i][1] = row_sum<RW>(ay[i][1]);
+    }
+    const int item = rtid / RW, lane_r = rtid % RW;
+    const int nT = (n_o + TI - 1) / TI;
+    const int nWin = (M_o + 1) >> 1;
+    if (item < nT * nWin) {
+        const int w = item % nWin, to = item / nWin;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int mo = 2 * w + k;
+            if (lane_r == (k % RW) && mo < M_o) {
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    const int ch = to + nT * i;
+                    if (ch < n_o) dst[ch * M_o + mo] = make_float2(ax[i][k], ay[i][k]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+}
+
+#define CGNET_BWD_SWITCH(TI_, RW_, CALL)                                         \
+    switch ((TI_) * 32 + (RW_)) {                                                \
+        case 1 * 32 + 1: { CALL(1, 1); } break;                                  \
+        case 1 * 32 + 2: { CALL(1, 2); } break;                                  \
+        case 1 * 32 + 4: { CALL(1, 4); } break;                                  \
+        case 1 * 32 + 8: { CALL(1, 8); } break;                                  \
+        case 1 * 32 + 16: { CALL(1, 16); } break;                                \
+        case 2 * 32 + 1: { CALL(2, 1); } break;                                  \
+        case 2 * 32 + 2: { CALL(2, 2); } break;                                  \
+        case 2 * 32 + 4: { CALL(2, 4); } break;                                  \
+        case 2 * 32 + 8: { CALL(2, 8); } break;                                  \
+        case 2 * 32 + 16: { CALL(2, 16); } break;                                \
+        case 3 * 32 + 1: { CALL(3, 1); } break;                                  \
+        case 3 * 32 + 2: { CALL(3, 2); } break;                                  \
+        case 3 * 32 + 4: { CALL(3, 4); } break;                                  \
+        case 3 * 32 + 8: { CALL(3, 8); } break;                                  \
+        case 3 * 32 + 16: { CALL(3, 16); } break;                                \
+        case 4 * 32 + 1: { CALL(4, 1); } break;                                  \
+        case 4 * 32 + 2: { CALL(4, 2); } break;                                  \
+        case 4 * 32 + 4: { CALL(4, 4); } break;                                  \
+        case 4 * 32 + 8: { CALL(4, 8); } break;                                  \
+        default: { CALL(4, 16); } break;                                         \
+    }
+
+// Registers that carry the next task's operands while the current task computes.
+constexpr int kPreTile = 8;   // gFF tile elements per thread   (covers 8 * 256 = 2048 complex = 16 KB)
+constexpr int kPreCg = 4;     // CG table entries per thread
+constexpr int kPreF = 2;      // fragment entries per thread
+struct BwdPrefetch {
+    float2 tile[kPreTile];
+    float cg[kPreCg];
+    float2 f2[kPreF];
+};
+
+// Issues the loads of task t (tile with zero padding along m, padded CG table, slab of degree l2).
+__device__ __forceinline__ void bwd_prefetch(BwdPrefetch& pf, const BwdUTask& t, int rows,
+                                             const float2* __restrict__ Gb, const float2* __restrict__ Fb,
+                                             const float* __restrict__ CG, int tid) {
+    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
+    const int Mp = M + kPadLo + kPadHi;
+    const int ntile = rows * t.tau2 * Mp;
+    const float inv = 1.0f / (float)Mp;
+    const float2* src = Gb + t.offFF;
+#pragma unroll
+    for (int k = 0; k < kPreTile; ++k) {
+        const int e = tid + k * kThreads;
+        const int ch = (int)(((float)e + 0.5f) * inv);
+        const int x = e - ch * Mp - kPadLo;
+        pf.tile[k] = make_float2(0.f, 0.f);
+        if (e < ntile && x >= 0 && x < M) pf.tile[k] = src[ch * M + x];
+    }
+    const int ncg = Mp * M2;
+#pragma unroll
+    for (int k = 0; k < kPreCg; ++k) {
+        const int e = tid + k * kThreads;
+        const int x = e - kPadLo * M2;
+        pf.cg[k] = 0.f;
+        if (e < ncg && x >= 0 && x < M * M2) pf.cg[k] = CG[t.cg_off + x];
+    }
+    if (t.first_of_l2) {
+        const int n2 = t.tau2 * M2;
+#pragma unroll
+        for (int k = 0; k < kPreF; ++k) {
+            const int e = tid + k * kThreads;
+            pf.f2[k] = make_float2(0.f, 0.f);
+            if (e < n2) pf.f2[k] = Fb[t.offF2 + e];
+        }
+    }
+}
+
+// Writes the prefetched operands of task t into LDS; entries beyond the register window are
+// loaded here directly (large shapes only).
+__device__ __forceinline__ void bwd_commit(const BwdPrefetch& pf, const BwdUTask& t, int rows,
+                                           const float2* __restrict__ Gb, const float2* __restrict__ Fb,
+                                           const float* __restrict__ CG, int tid,
+                                           float2* __restrict__ f2, float* __restrict__ cgp, float2* __restrict__ g) {
+    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
+    const int Mp = M + kPadLo + kPadHi;
+    const int ntile = rows * t.tau2 * Mp, ncg = Mp * M2, n2 = t.tau2 * M2;
+#pragma unroll
+    for (int k = 0; k < kPreTile; ++k) {
+        const int e = tid + k * kThreads;
+        if (e < ntile) g[e] = pf.tile[k];
+    }
+#pragma unroll
+    for (int k = 0; k < kPreCg; ++k) {
+        const int e = tid + k * kThreads;
+        if (e < ncg) cgp[e] = pf.cg[k];
+    }
+    if (t.first_of_l2) {
+#pragma unroll
+        for (int k = 0; k < kPreF; ++k) {
+            const int e = tid + k * kThreads;
+            if (e < n2) f2[e] = pf.f2[k];
+        }
+        for (int e = tid + kPreF * kThreads; e < n2; e += kThreads) f2[e] = Fb[t.offF2 + e];
+    }
+    if (ntile > kPreTile * kThreads) {
+        const float inv = 1.0f / (float)Mp;
+        const float2* src = Gb + t.offFF;
+        for (int e = tid + kPreTile * kThreads; e < ntile; e += kThreads) {
+            const int ch = (int)(((float)e + 0.5f) * inv);
+            const int x = e - ch * Mp - kPadLo;
+            float2 v = make_float2(0.f, 0.f);
+            if (x >= 0 && x < M) v = src[ch * M + x];
+            g[e] = v;
+        }
+    }
+    for (int e = tid + kPreCg * kThreads; e < ncg; e += kThreads) {
+        const int x = e - kPadLo * M2;
+        cgp[e] = (x >= 0 && x < M * M2) ? CG[t.cg_off + x] : 0.f;
+    }
+}
+
+struct BwdCtx {
+    const float2* Fb;          // this sample's fragments
+    const float2* Gb;          // this sample's gFF
+    const float* CG;
+    const BwdUTask* tasks;
+    float2* f1;                // LDS: rows x M1 slab of degree l1 (fixed for the unit)
+    float2* f2;                // LDS: slab of the current l2, followed by the CG table and the tile
+    int tid, rtid;
+};
+
+// Common per-task prologue of both roles: publish the prefetched operands of task `t` in LDS and
+// start loading the next task's.  Every thread of the group executes the two barriers.
+__device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int ti, BwdPrefetch& pf,
+                                          BwdUTask& t, BwdUTask& cur, float*& cgp, float2*& g) {
+    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
+    const int Mp = M + kPadLo + kPadHi;
+    cgp = reinterpret_cast<float*>(c.f2 + t.tau2 * M2);
+    g = reinterpret_cast<float2*>(cgp + ((Mp * M2 + 1) & ~1));
+    __syncthreads();                                 // the previous tile (and f2) are no longer read
+    bwd_commit(pf, t, u.rows, c.Gb, c.Fb, c.CG, c.tid, c.f2, cgp, g);
+    __syncthreads();
+    cur = t;
+    if (ti + 1 < u.task_end) {                       // next task's loads fly while this one computes
+        t = c.tasks[ti + 1];
+        bwd_prefetch(pf, t, u.rows, c.Gb, c.Fb, c.CG, c.tid);
+    }
+}
+
+// Waves of role A: gradient of slot 1 (rows of degree l1), kept in registers for the whole unit.
+template <int TI, int RW>
+__device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
+                                                float2* __restrict__ dst) {
+    float ax[4][2], ay[4][2], tx[4][2], ty[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+        tx[i][0] = tx[i][1] = ty[i][0] = ty[i][1] = 0.f;
+    }
+    for (int ti = u.task_begin; ti < u.task_end; ++ti) {
+        BwdUTask cur;
+        float* cgp;
+        float2* g;
+        bwd_stage(c, u, ti, pf, t, cur, cgp, g);
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+        bwd_accum<1, TI, RW>(q, cgp, g, c.f2, c.rtid, ax, ay);
+        if (cur.last_of_l2) {
+            // blocked summation: the running sum of one l2 is folded into the unit's total
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    tx[i][k] += ax[i][k];
+                    ty[i][k] += ay[i][k];
+                    ax[i][k] = ay[i][k] = 0.f;
+                }
+        }
+    }
+    bwd_flush<TI, RW>(u.rows, 2 * u.l1 + 1, c.rtid, tx, ty, dst);
+}
+
+// Waves of role B: gradient of slot 2, kept in registers across the tasks that share l2.
+__device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
+                                                float2* __restrict__ part2_b) {
+    float ax[4][2], ay[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+    for (int ti = u.task_begin; ti < u.task_end; ++ti) {
+        BwdUTask cur;
+        float* cgp;
+        float2* g;
+        bwd_stage(c, u, ti, pf, t, cur, cgp, g);
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+#define CGNET_CALL_B(TI_, RW_) bwd_accum<2, TI_, RW_>(q, cgp, g, c.f1, c.rtid, ax, ay)
+        CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_CALL_B)
+#undef CGNET_CALL_B
+        if (cur.last_of_l2) {
+            float2* dst = part2_b + cur.p2off;
+#define CGNET_FLUSH_B(TI_, RW_) bwd_flush<TI_, RW_>(cur.tau2, 2 * cur.l2 + 1, c.rtid, ax, ay, dst)
+            CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_FLUSH_B)
+#undef CGNET_FLUSH_B
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kThreads, 3)
+cg_backward_unit_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
+                        const float* __restrict__ CG, float2* __restrict__ part1, float2* __restrict__ part2,
+                        const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
+                        int nF, int nFF, int P2) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const BwdUnit u = units[blockIdx.x];
+    const int b = blockIdx.y;
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const int M1 = 2 * u.l1 + 1;
+    const bool roleA = wave < u.nA;                  // wave-uniform
+    BwdCtx c;
+    c.Fb = F + (size_t)b * nF;
+    c.Gb = gFF + (size_t)b * nFF;
+    c.CG = CG;
+    c.tasks = tasks;
+    c.f1 = reinterpret_cast<float2*>(smem);
+    c.f2 = c.f1 + u.rows * M1;
+    c.tid = tid;
+    c.rtid = roleA ? tid : tid - 64 * u.nA;
+
+    BwdPrefetch pf;
+    const BwdUTask t0 = tasks[u.task_begin];
+    bwd_prefetch(pf, t0, u.rows, c.Gb, c.Fb, CG, tid);
+    for (int e = tid; e < u.rows * M1; e += kThreads) c.f1[e] = c.Fb[u.offF1 + e];
+
+    // The two roles run the same sequence of barriers (two per task) from different code paths.
+    if (roleA) {
+        float2* dst = part1 + (size_t)b * nF + u.offF1;
+#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<TI_, RW_>(c, u, pf, t0, dst)
+        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#undef CGNET_LOOP_A
+    } else {
+        bwd_unit_loop_b(c, u, pf, t0, part2 + (size_t)b * P2);
+    }
+}
+
+// gF[b][e] = slot-1 part (if any unit owns the degree) + the slot-2 slabs of that degree, in list order
+__global__ void __launch_bounds__(256)
+cg_backward_combine_kernel(const float2* __restrict__ part1, const float2* __restrict__ part2,
+                           float2* __restrict__ gF, const int* __restrict__ meta, int L, int nF, int P2, int B) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)B * nF) return;
+    const int b = (int)(idx / nF), e = (int)(idx % nF);
+    const int* cumF = meta;                 // L+2
+    const int* own1 = meta + (L + 2);       // L+1
+    const int* lbeg = own1 + (L + 1);       // L+2
+    const int* loff = lbeg + (L + 2);
+    int lam = 0;
+    while (lam < L && cumF[lam + 1] <= e) ++lam;
+    const int rel = e - cumF[lam];
+    float2 s = make_float2(0.f, 0.f);
+    if (own1[lam]) s = part1[idx];
+    const float2* p2 = part2 + (size_t)b * P2;
+    for (int k = lbeg[lam]; k < lbeg[lam + 1]; ++k) {
+        const float2 v = p2[loff[k] + rel];
+        s.x += v.x;
+        s.y += v.y;
+    }
+    gF[idx] = s;
 }
 
 __global__ void __launch_bounds__(256)
@@ -395,6 +889,9 @@ static void free_plan(cgnet_cg_plan* plan) {
     if (plan->d_fwd_tasks) (void)hipFree(plan->d_fwd_tasks);
     if (plan->d_bwd_tasks) (void)hipFree(plan->d_bwd_tasks);
     if (plan->d_bwd_group_table) (void)hipFree(plan->d_bwd_group_table);
+    if (plan->d_bwd_units) (void)hipFree(plan->d_bwd_units);
+    if (plan->d_bwd_utasks) (void)hipFree(plan->d_bwd_utasks);
+    if (plan->d_bwd_combine) (void)hipFree(plan->d_bwd_combine);
     delete plan;
 }
 
@@ -457,13 +954,13 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     p->nFF = p->cumFF[n1];
     p->sumT = p->cumT[n1];
 
-    auto build = [&](int tile_bytes, std::vector<CgTask>* out) -> int {
+    auto build = [&](int tile_bytes, std::vector<CgTask>* out, int pad = 0) -> int {
         for (int i = 0; i < nllls; ++i) {
             const int l = tl[i], l1 = tl1[i], l2 = tl2[i];
             const int tau1 = h_t_F[l1], tau2 = h_t_F[l2];
             if (tau1 == 0 || tau2 == 0) continue;
             const int M = 2 * l + 1;
-            const long long row_bytes = 8LL * tau2 * M;
+            const long long row_bytes = 8LL * tau2 * (M + pad);
             int max_rows = (int)std::min<long long>(tau1, std::max<long long>(1, tile_bytes / row_bytes));
             max_rows = std::max(1, std::min(max_rows, kMaxTileChannels / tau2));
             const int nchunks = (tau1 + max_rows - 1) / max_rows;
@@ -482,13 +979,52 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 t.TI = (t.rows + t.nT1 - 1) / t.nT1;
                 t.nT2 = (tau2 + 3) / 4;
                 t.TJ = (tau2 + t.nT2 - 1) / t.nT2;
+                t.bTI[0] = t.bTI[1] = 1;
+                t.bRW[0] = t.bRW[1] = 1;
                 out->push_back(t);
             }
         }
         return 0;
     };
     build(kFwdTileBytes, &p->fwd_tasks);
-    build(kBwdTileBytes, &p->bwd_tasks);
+    p->bwd_tasks.clear();
+    build(kBwdTileBytes, &p->bwd_tasks, kPadLo + kPadHi);
+    // Backward tiling.  Per slot a thread owns TI output channels x 2 m and RW lanes split the
+    // reduced channels.  cost = passes over the work-group * sequential steps of a lane * TI;
+    // the work-group size that wastes the fewest lane-steps over all tasks is kept.
+    {
+        const int cand[3] = {128, 192, 256};
+        double best_total = -1;
+        for (int ci = 0; ci < 3; ++ci) {
+            const int wg = cand[ci];
+            double total = 0;
+            std::vector<CgTask> tmp = p->bwd_tasks;
+            for (CgTask& t : tmp) {
+                for (int slot = 0; slot < 2; ++slot) {
+                    const int n_o = slot == 0 ? t.rows : t.tau2, n_r = slot == 0 ? t.tau2 : t.rows;
+                    const int M_o = slot == 0 ? 2 * t.l1 + 1 : 2 * t.l2 + 1;
+                    const int M_r = slot == 0 ? 2 * t.l2 + 1 : 2 * t.l1 + 1;
+                    double best = -1;
+                    for (int ti = 1; ti <= 4; ++ti)
+                        for (int rw = 1; rw <= 16; rw *= 2) {
+                            if (rw > 1 && rw / 2 >= n_r) continue;
+                            const int items = ((n_o + ti - 1) / ti) * ((M_o + 1) / 2);
+                            const int rows_blk = wg / rw;
+                            const double passes = (items + rows_blk - 1) / rows_blk;
+                            // steps of one lane; the row reduction costs about 2*ti*log2(rw) more
+                            double c = passes * (((n_r + rw - 1) / rw) * (double)M_r * (ti + 0.75) + 1.5 * ti * rw);
+                            if (best < 0 || c < best) { best = c; t.bTI[slot] = ti; t.bRW[slot] = rw; }
+                        }
+                    total += best * wg;
+                }
+            }
+            if (best_total < 0 || total < best_total) {
+                best_total = total;
+                p->bwd_threads = wg;
+                p->bwd_tasks = tmp;
+            }
+        }
+    }
     // heaviest forward tasks first: a short tail when the grid drains
     std::stable_sort(p->fwd_tasks.begin(), p->fwd_tasks.end(), [](const CgTask& a, const CgTask& b) {
         return (long long)a.rows * a.tau2 * (2 * a.l + 1) * (2 * a.l2 + 1) >
@@ -496,7 +1032,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     });
     size_t fl = 0, bl = 0;
     for (const CgTask& t : p->fwd_tasks) fl = std::max(fl, fwd_task_lds(t));
-    for (const CgTask& t : p->bwd_tasks) bl = std::max(bl, fwd_task_lds(t));
+    for (const CgTask& t : p->bwd_tasks) bl = std::max(bl, bwd_task_lds(t));
     p->fwd_lds = align_up(fl, 16);
     p->bwd_lds = align_up(bl, 16) + 8 * (size_t)p->nF;
     CGNET_REQUIRE(p->fwd_lds <= kMaxLds, CGNET_ERR_UNSUPPORTED,
@@ -539,6 +1075,153 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         }
     }
 
+    // ---- register-resident backward: units = (l1, range of t1 rows), tasks ordered by (l2, l)
+    std::vector<int> combine_meta;
+    {
+        bool ok = true;
+        int P2 = 0;
+        size_t lds_max = 0;
+        std::vector<int> own1(n1, 0);
+        std::vector<std::vector<int>> lam_offs(n1);
+        std::vector<double> unit_cost;
+        for (int l1 = 0; l1 < n1 && ok; ++l1) {
+            std::vector<int> tri;
+            for (int i = 0; i < nllls; ++i)
+                if (tl1[i] == l1 && h_t_F[l1] > 0 && h_t_F[tl2[i]] > 0) tri.push_back(i);
+            if (tri.empty()) continue;
+            own1[l1] = 1;
+            std::stable_sort(tri.begin(), tri.end(), [&](int a, int b) {
+                return tl2[a] != tl2[b] ? tl2[a] < tl2[b] : tl[a] < tl[b];
+            });
+            const int tau1 = h_t_F[l1], M1 = 2 * l1 + 1;
+            const int nt = (int)tri.size();
+            struct Choice { double total = -1; int rows = 0, nA = 0, TI = 0, RW = 0; std::vector<int> bTI, bRW; };
+            Choice best;
+            int prev_rows = -1;
+            for (int nchunks = 1; nchunks <= tau1; ++nchunks) {
+                const int rows_c = (tau1 + nchunks - 1) / nchunks;
+                if (rows_c == prev_rows) continue;
+                prev_rows = rows_c;
+                long long max_tile = 0;
+                for (int i : tri) max_tile = std::max(max_tile, 8LL * rows_c * h_t_F[tl2[i]] * (2 * tl[i] + 1 + kPadLo + kPadHi));
+                if (max_tile > kBwdTileBytes && rows_c > 1) continue;
+                const int real_chunks = (tau1 + rows_c - 1) / rows_c;
+                for (int nA = 1; nA <= 3; ++nA) {
+                    const int lanesA = 64 * nA, lanesB = kThreads - lanesA;
+                    // slot 2: best tiling per task (constant within a run of equal l2)
+                    std::vector<double> costB(nt);
+                    std::vector<int> bTI(nt), bRW(nt);
+                    bool feasible = true;
+                    for (int k = 0; k < nt && feasible; ++k) {
+                        const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
+                        double bc = -1;
+                        for (int ti = 1; ti <= 4; ++ti)
+                            for (int rw = 1; rw <= 16; rw *= 2) {
+                                if (rw > 1 && rw / 2 >= rows_c) continue;
+                                const int items = ((tau2 + ti - 1) / ti) * ((M2 + 1) / 2);
+                                if (items * rw > lanesB) continue;
+                                const double c = ((rows_c + rw - 1) / rw) * (double)M1 * (8.0 * ti + 14.0);
+                                if (bc < 0 || c < bc) { bc = c; bTI[k] = ti; bRW[k] = rw; }
+                            }
+                        if (bc < 0) feasible = false;
+                        costB[k] = bc;
+                    }
+                    if (!feasible) continue;
+                    int max_tau2 = 1;
+                    for (int i : tri) max_tau2 = std::max(max_tau2, h_t_F[tl2[i]]);
+                    for (int ti = 1; ti <= 4; ++ti)
+                        for (int rw = 1; rw <= 16; rw *= 2) {
+                            if (rw > 1 && rw / 2 >= max_tau2) continue;
+                            const int items = ((rows_c + ti - 1) / ti) * ((M1 + 1) / 2);
+                            if (items * rw > lanesA) continue;
+                            double total = 0;
+                            for (int k = 0; k < nt; ++k) {
+                                const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
+                                const double cA = ((tau2 + rw - 1) / rw) * (double)M2 * (8.0 * ti + 14.0);
+                                const double stage = 12.0 * rows_c * tau2 * (2 * tl[tri[k]] + 4) / kThreads + 200.0;
+                                total += std::max(cA, costB[k]) + stage;
+                            }
+                            total *= real_chunks;
+                            if (best.total < 0 || total < best.total) {
+                                best.total = total; best.rows = rows_c; best.nA = nA; best.TI = ti; best.RW = rw;
+                                best.bTI = bTI; best.bRW = bRW;
+                            }
+                        }
+                }
+            }
+            if (best.total < 0) { ok = false; break; }
+            for (int r0 = 0; r0 < tau1; r0 += best.rows) {
+                BwdUnit u;
+                u.l1 = l1;
+                u.rows = std::min(best.rows, tau1 - r0);
+                u.offF1 = p->cumF[l1] + r0 * M1;
+                u.task_begin = (int)p->bwd_utasks.size();
+                u.nA = best.nA; u.TI = best.TI; u.RW = best.RW;
+                size_t task_lds = 0;
+                for (int k = 0; k < nt; ++k) {
+                    const int i = tri[k];
+                    BwdUTask t;
+                    t.l = tl[i]; t.l2 = tl2[i]; t.tau2 = h_t_F[tl2[i]];
+                    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1, Mp = M + kPadLo + kPadHi;
+                    t.offFF = p->cumFF[t.l] + (p->t_off[i] + r0 * t.tau2) * M;
+                    t.offF2 = p->cumF[t.l2];
+                    t.cg_off = cgo[i];
+                    t.first_of_l2 = (k == 0 || tl2[tri[k - 1]] != t.l2) ? 1 : 0;
+                    t.last_of_l2 = (k + 1 == nt || tl2[tri[k + 1]] != t.l2) ? 1 : 0;
+                    if (t.first_of_l2) {
+                        lam_offs[t.l2].push_back(P2);
+                        t.p2off = P2;
+                        P2 += t.tau2 * M2;
+                    } else {
+                        t.p2off = p->bwd_utasks.back().p2off;
+                    }
+                    t.TI = best.bTI[k]; t.RW = best.bRW[k];
+                    p->bwd_utasks.push_back(t);
+                    task_lds = std::max(task_lds, (size_t)8 * t.tau2 * M2 + 4 * (size_t)((Mp * M2 + 1) & ~1) +
+                                                      (size_t)8 * u.rows * t.tau2 * Mp);
+                }
+                u.task_end = (int)p->bwd_utasks.size();
+                lds_max = std::max(lds_max, (size_t)8 * u.rows * M1 + task_lds);
+                p->bwd_units.push_back(u);
+                unit_cost.push_back(best.total);
+            }
+        }
+        // CGNET_BWD_GENERAL=1 forces the LDS-accumulator kernel (kept for shapes the unit scheme cannot hold)
+        const char* force_general = getenv("CGNET_BWD_GENERAL");
+        if (force_general && force_general[0] == '1') ok = false;
+        if (ok && !p->bwd_units.empty() && lds_max <= kMaxLds) {
+            // longest units first
+            std::vector<int> order(p->bwd_units.size());
+            for (size_t k = 0; k < order.size(); ++k) order[k] = (int)k;
+            std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return unit_cost[a] > unit_cost[b]; });
+            std::vector<BwdUnit> sorted;
+            for (int k : order) sorted.push_back(p->bwd_units[k]);
+            p->bwd_units.swap(sorted);
+            p->bwd_fast = true;
+            p->bwd_P2 = P2;
+            if (const char* dbg = getenv("CGNET_DEBUG"); dbg && dbg[0] == '1') {
+                fprintf(stderr, "[cgnet] backward units=%zu tasks=%zu P2=%d lds=%zu\n", p->bwd_units.size(),
+                        p->bwd_utasks.size(), P2, lds_max);
+                for (const BwdUnit& u : p->bwd_units) {
+                    const BwdUTask& t0 = p->bwd_utasks[u.task_begin];
+                    const BwdUTask& t1 = p->bwd_utasks[u.task_end - 1];
+                    fprintf(stderr, "[cgnet]   l1=%d rows=%d tasks=%d nA=%d A(TI=%d,RW=%d) B first(TI=%d,RW=%d) last(TI=%d,RW=%d)\n",
+                            u.l1, u.rows, u.task_end - u.task_begin, u.nA, u.TI, u.RW, t0.TI, t0.RW, t1.TI, t1.RW);
+                }
+            }
+            p->bwd_fast_lds = align_up(lds_max, 16);
+            combine_meta.insert(combine_meta.end(), p->cumF.begin(), p->cumF.end());   // L+2
+            combine_meta.insert(combine_meta.end(), own1.begin(), own1.end());         // L+1
+            int run = 0;
+            for (int l = 0; l < n1; ++l) { combine_meta.push_back(run); run += (int)lam_offs[l].size(); }
+            combine_meta.push_back(run);
+            for (int l = 0; l < n1; ++l) combine_meta.insert(combine_meta.end(), lam_offs[l].begin(), lam_offs[l].end());
+        } else {
+            p->bwd_units.clear();
+            p->bwd_utasks.clear();
+        }
+    }
+
     CGNET_HIP(hipGetDevice(&p->device));
     if (!p->fwd_tasks.empty()) {
         CGNET_HIP(hipMalloc((void**)&p->d_fwd_tasks, sizeof(CgTask) * p->fwd_tasks.size()));
@@ -547,6 +1230,16 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         CGNET_HIP(hipMemcpy(p->d_bwd_tasks, p->bwd_tasks.data(), sizeof(CgTask) * p->bwd_tasks.size(), hipMemcpyHostToDevice));
         CGNET_HIP(hipMalloc((void**)&p->d_bwd_group_table, sizeof(int) * gtab.size()));
         CGNET_HIP(hipMemcpy(p->d_bwd_group_table, gtab.data(), sizeof(int) * gtab.size(), hipMemcpyHostToDevice));
+    }
+    if (p->bwd_fast) {
+        CGNET_HIP(hipMalloc((void**)&p->d_bwd_units, sizeof(BwdUnit) * p->bwd_units.size()));
+        CGNET_HIP(hipMemcpy(p->d_bwd_units, p->bwd_units.data(), sizeof(BwdUnit) * p->bwd_units.size(), hipMemcpyHostToDevice));
+        CGNET_HIP(hipMalloc((void**)&p->d_bwd_utasks, sizeof(BwdUTask) * p->bwd_utasks.size()));
+        CGNET_HIP(hipMemcpy(p->d_bwd_utasks, p->bwd_utasks.data(), sizeof(BwdUTask) * p->bwd_utasks.size(), hipMemcpyHostToDevice));
+        CGNET_HIP(hipMalloc((void**)&p->d_bwd_combine, sizeof(int) * combine_meta.size()));
+        CGNET_HIP(hipMemcpy(p->d_bwd_combine, combine_meta.data(), sizeof(int) * combine_meta.size(), hipMemcpyHostToDevice));
+        if (p->bwd_fast_lds > 64 * 1024)
+            CGNET_HIP(hipFuncSetAttribute((const void*)cg_backward_unit_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_fast_lds));
     }
     if (p->fwd_lds > 64 * 1024)
         CGNET_HIP(hipFuncSetAttribute((const void*)cg_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->fwd_lds));
@@ -641,6 +1334,9 @@ extern "C" int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float
 
 extern "C" size_t cgnet_sparse_backward_workspace(const cgnet_cg_plan* plan, int B) {
     if (!plan || B <= 0) return 0;
+    if (plan->bwd_fast)
+        return align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256) +
+               align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256);
     const int ng = bwd_groups_for(plan, B);
     if (ng <= 1) return 0;
     return align_up(sizeof(float) * 2 * (size_t)plan->nF * B * ng, 256);
@@ -666,11 +1362,25 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
     const size_t need = cgnet_sparse_backward_workspace(plan, B);
     CGNET_REQUIRE(need == 0 || (d_workspace && workspace_bytes >= need), CGNET_ERR_WORKSPACE,
                   "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if (plan->bwd_fast) {
+        float2* part1 = (float2*)d_workspace;
+        float2* part2 = (float2*)((char*)d_workspace + align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256));
+        CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)plan->bwd_units.size(), B), dim3(kThreads),
+                     plan->bwd_fast_lds, s, (const float2*)d_F, (const float2*)d_gFF, d_CG, part1, part2,
+                     plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->nFF, plan->bwd_P2);
+        CGNET_HIP(hipGetLastError());
+        const size_t n = (size_t)plan->nF * B;
+        CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+                     (const float2*)part1, (const float2*)part2, (float2*)d_gF, plan->d_bwd_combine, plan->L,
+                     plan->nF, plan->bwd_P2, B);
+        CGNET_HIP(hipGetLastError());
+        return CGNET_OK;
+    }
     const int* d_gb = plan->d_bwd_group_table + plan->bwd_group_table_off[ng];
     float2* dst = ng > 1 ? (float2*)d_workspace : (float2*)d_gF;
-    CGNET_LAUNCH(cg_backward_kernel, dim3(ng, B), dim3(kThreads), plan->bwd_lds, s,
+    CGNET_LAUNCH(cg_backward_kernel, dim3(ng, B), dim3(plan->bwd_threads), plan->bwd_lds, s,
                        (const float2*)d_F, (const float2*)d_gFF, d_CG, dst, plan->d_bwd_tasks, d_gb,
-                       plan->nF, plan->nFF, B, 0);
+                       plan->nF, plan->nFF, B);
     CGNET_HIP(hipGetLastError());
     if (ng > 1) {
         const size_t n = (size_t)plan->nF * B;

@@ -135,6 +135,28 @@ def test_cg_forward_backward(dev, lmax, taus, bsz, mode):
     assert torch.equal(torch.cat([p.reshape(bsz, -1, 2) for p in y_list], 1), y.detach())
 
 
+@pytest.mark.parametrize("lmax,taus,bsz,mode", [CG_CASES[2], CG_CASES[5], CG_CASES[7]])
+def test_cg_backward_general_kernel(dev, monkeypatch, lmax, taus, bsz, mode):
+    """The LDS-accumulator backward kernel (fallback for shapes the register-resident scheme cannot
+    hold) is forced through the CGNET_BWD_GENERAL switch, read when a plan is created."""
+    from cgnet_amd import _plans
+    monkeypatch.setenv("CGNET_BWD_GENERAL", "1")
+    codes = make_codes(lmax, mode)
+    plan = _plans.CGPlan(lmax, taus, codes)
+    monkeypatch.delenv("CGNET_BWD_GENERAL")
+    _, offs = OC.flat_cg_table(OT.decode(lmax, codes), dtype=np.float32)
+    cg = torch.zeros(int(offs[-1]), device=dev)
+    _plans.fill_cg_table(cg, lmax, codes, [int(v) for v in offs])
+    x64 = rand_straight(taus, bsz, seed=77)
+    g = torch.Generator().manual_seed(78)
+    gy64 = torch.randn(bsz, plan.nFF, 2, generator=g, dtype=torch.float64)
+    _, want_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64)
+    x = x64.float().to(dev)
+    gx = torch.full_like(x, float("nan"))
+    plan.backward(x, gx, gy64.float().to(dev), cg, bsz)
+    assert_close(gx, want_gx, "CG backward (general kernel)")
+
+
 def test_cg_forward_matches_dense_definition(dev):
     # config 1 against the explicit six-index loop definition (independent of the oracle's matmul path)
     from oracle import bruteforce as BF
