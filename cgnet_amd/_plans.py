@@ -28,6 +28,11 @@ def _require_gpu(name, t, dtype=torch.float32):
         raise RuntimeError("%s must have dtype %s (got %s)" % (name, dtype, t.dtype))
 
 
+def _aligned16(t):
+    """The streaming kernels use 16-byte loads; a view that starts mid-allocation is copied."""
+    return t if t is None or t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
@@ -187,6 +192,9 @@ class WMMPlan:
                 or (gFF is not None and gFF.numel() != FF.numel()) or (gW is not None and gW.numel() != W.numel())):
             raise RuntimeError("FN_WMM_backward: tensor sizes do not match the plan")
         lib = _lib.load()
+        gO, FF = _aligned16(gO), _aligned16(FF)
+        if gFF is not None and gFF.data_ptr() % 16:
+            raise RuntimeError("grad_FF must be 16-byte aligned")
         with torch.cuda.device(FF.device):
             ws = _workspace(lib.cgnet_FN_WMM_backward_workspace(self._h, int(B)), FF.device)
             _lib.check(lib.cgnet_FN_WMM_backward(self._h, _ptr(gO), _ptr(gFF), _ptr(gW), _ptr(FF), _ptr(W), int(B),

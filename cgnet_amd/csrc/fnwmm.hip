@@ -34,6 +34,8 @@ struct WmmDeg {
     int wp_base;       // first 64-float block of the degree in the packed weights
     int G, NC;         // forward: samples per work-group, 32-column chunks per wave
     int S;             // forward: number of k-slices
+    int nks_b;         // gradient wrt FF: k-steps of 4 over the 2*tO real rows (re, im interleaved)
+    int ap_base;       // first 64-float block of the degree in the packed conj(W)/div operand
 };
 
 struct WmmFwdUnit { int deg, rc, slice, k_begin, k_end; };
@@ -45,14 +47,20 @@ struct cgnet_wmm_plan {
     int L = 0;
     int nFF = 0, nO = 0, nW = 0, sumT = 0;
     int wp_blocks = 0;     // 64-float blocks of the packed forward weights
+    int ap_blocks = 0;     // 64-float blocks of the packed operand of the FF-gradient kernel
+    bool gff_mfma = true;  // every degree has t_O <= 16 (the operand then fits eight registers)
+    int gw_ff_cap = 2, gw_go_cap = 2;   // LDS capacities (complex entries) of one stage of the weight-gradient kernel
+    int fwd_stage_cap = 2;              // LDS capacity (complex entries) of one stage of the forward kernel
+    int gff_out_cap = 4, gff_go_cap = 2; // LDS capacities of the FF-gradient kernel (real entries / complex entries)
     int maxS = 1, maxG = 1;
     std::vector<cgnet::WmmDeg> degs;
     std::vector<cgnet::WmmFwdUnit> fwd_units;
-    std::vector<cgnet::WmmChanUnit> gw_units, gff_units, stat_units;
+    std::vector<cgnet::WmmChanUnit> gw_units, gw_units_rc0, gff_units, stat_units;
     std::vector<int> cumO_all, cumFF_all;   // L+2 entries, for element -> degree lookups
     cgnet::WmmDeg* d_degs = nullptr;
     cgnet::WmmFwdUnit* d_fwd_units = nullptr;
     cgnet::WmmChanUnit* d_gw_units = nullptr;
+    cgnet::WmmChanUnit* d_gw_units_rc0 = nullptr;   // one entry per 64-channel chunk (row chunk 0 only)
     cgnet::WmmChanUnit* d_gff_units = nullptr;
     cgnet::WmmChanUnit* d_stat_units = nullptr;
     int* d_cumO = nullptr;      // per deg index: cumO, and S, interleaved: [ndeg+1] cumO then [ndeg] S
@@ -190,114 +198,192 @@ __device__ __forceinline__ void mfma_drain() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int NC>
-__device__ __forceinline__ void wmm_forward_body(const float* __restrict__ FF, const float* __restrict__ Wp,
-                                                 float2* __restrict__ out, const WmmDeg& d,
-                                                 const WmmFwdUnit& u, int B, int nFF, int nO, f32x4 (*red)[8][64]) {
-    const int b0 = blockIdx.y * d.G;
-    if (b0 >= B) return;
-    const int nb = min(d.G, B - b0);
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int i = lane & 15, kk = lane >> 4;
-    const int M = d.M, n2 = 2 * d.M;
-    const int ncols = nb * M;
-
-    size_t off[NC][2];
-    bool ok[NC][2];
+// Streaming helper: a contiguous run of n complex numbers starting at element `off` of a
+// (16-byte aligned) float2 array is fetched with 16-byte loads, lane-contiguous, from the
+// element pair that contains `off`; the LDS image therefore starts `off & 1` elements early.
+template <int NREG>
+struct Run16 {
+    float4 r[NREG];
+    // issue the loads (whole work-group, tid = 0..nthreads-1); elements beyond `total` are not touched
+    __device__ __forceinline__ void fetch(const float2* __restrict__ base, size_t off, int n, size_t total, int tid,
+                                          int nthreads) {
+        const size_t first = off & ~(size_t)1;
+        const int n4 = (n + (int)(off & 1) + 1) >> 1;
+        const float4* src = reinterpret_cast<const float4*>(base + first);
 #pragma unroll
-    for (int nc = 0; nc < NC; ++nc)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int q = nc * 32 + 2 * i + h;
-            ok[nc][h] = q < ncols;
-            const int bl = ok[nc][h] ? q / M : 0;
-            const int m = ok[nc][h] ? q - bl * M : 0;
-            off[nc][h] = ((size_t)(b0 + bl) * nFF + d.cumFF + m) * 2;
-        }
-
-    f32x4 acc[2][NC * 4];
-#pragma unroll
-    for (int t = 0; t < NC * 4; ++t) {
-        acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        acc[1][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
-    const int nsteps = (u.k_end - u.k_begin + 3) >> 2;
-    const int ks0 = u.k_begin >> 2;
-    for (int s = w; s < nsteps; s += 4) {
-        const int k = u.k_begin + 4 * s + kk;
-        const bool kin = k < u.k_end;
-        const float* ap = Wp + ((size_t)(d.wp_base + ((ks0 + s) * d.nrc + u.rc) * 2)) * 64 + lane;
-        const float a0 = ap[0], a1 = ap[64];
-        float2 bv[NC][2];
-#pragma unroll
-        for (int nc = 0; nc < NC; ++nc)
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                bv[nc][h] = make_float2(0.f, 0.f);
-                if (ok[nc][h] && kin) bv[nc][h] = *reinterpret_cast<const float2*>(FF + off[nc][h] + (size_t)k * n2);
-            }
-#pragma unroll
-        for (int nc = 0; nc < NC; ++nc) {
-            acc[0][nc * 4 + 0] = mfma4(a0, bv[nc][0].x, acc[0][nc * 4 + 0]);
-            acc[0][nc * 4 + 1] = mfma4(a0, bv[nc][0].y, acc[0][nc * 4 + 1]);
-            acc[0][nc * 4 + 2] = mfma4(a0, bv[nc][1].x, acc[0][nc * 4 + 2]);
-            acc[0][nc * 4 + 3] = mfma4(a0, bv[nc][1].y, acc[0][nc * 4 + 3]);
-            acc[1][nc * 4 + 0] = mfma4(a1, bv[nc][0].x, acc[1][nc * 4 + 0]);
-            acc[1][nc * 4 + 1] = mfma4(a1, bv[nc][0].y, acc[1][nc * 4 + 1]);
-            acc[1][nc * 4 + 2] = mfma4(a1, bv[nc][1].x, acc[1][nc * 4 + 2]);
-            acc[1][nc * 4 + 3] = mfma4(a1, bv[nc][1].y, acc[1][nc * 4 + 3]);
-        }
-    }
-
-    mfma_drain();
-    // add the four waves' partial sums in a fixed order, then form the complex outputs
-    float2* dst = out + (size_t)u.slice * B * nO;
-#pragma unroll
-    for (int nc = 0; nc < NC; ++nc) {
-        __syncthreads();
-        if (w > 0) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                red[w - 1][t][lane] = acc[0][nc * 4 + t];
-                red[w - 1][4 + t][lane] = acc[1][nc * 4 + t];
-            }
-        }
-        __syncthreads();
-        if (w == 0) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                acc[0][nc * 4 + t] = ((acc[0][nc * 4 + t] + red[0][t][lane]) + red[1][t][lane]) + red[2][t][lane];
-                acc[1][nc * 4 + t] = ((acc[1][nc * 4 + t] + red[0][4 + t][lane]) + red[1][4 + t][lane]) + red[2][4 + t][lane];
-            }
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                if (!ok[nc][h]) continue;
-                const int q = nc * 32 + 2 * i + h;
-                const int bl = q / M, m = q - bl * M;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int to = u.rc * 16 + 4 * kk + v;
-                    if (to < d.tO) {
-                        const float re = acc[0][nc * 4 + 2 * h][v] - acc[1][nc * 4 + 2 * h + 1][v];
-                        const float im = acc[0][nc * 4 + 2 * h + 1][v] + acc[1][nc * 4 + 2 * h][v];
-                        dst[(size_t)(b0 + bl) * nO + d.cumO + to * M + m] = make_float2(re, im);
-                    }
+        for (int k = 0; k < NREG; ++k) {
+            const int idx = tid + k * nthreads;
+            r[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (idx < n4) {
+                if (first + 2 * (size_t)idx + 1 < total) {
+                    r[k] = src[idx];
+                } else {
+                    const float2 z = base[first + 2 * (size_t)idx];
+                    r[k] = make_float4(z.x, z.y, 0.f, 0.f);
                 }
             }
         }
     }
-}
+    __device__ __forceinline__ void commit(float2* __restrict__ lds, size_t off, int n, int tid, int nthreads) const {
+        const int n4 = (n + (int)(off & 1) + 1) >> 1;
+        float4* dst = reinterpret_cast<float4*>(lds);
+#pragma unroll
+        for (int k = 0; k < NREG; ++k) {
+            const int idx = tid + k * nthreads;
+            if (idx < n4) dst[idx] = r[k];
+        }
+    }
+};
 
-__global__ void __launch_bounds__(kThreads)
-wmm_forward_kernel(const float* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
-                   const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO) {
-    __shared__ f32x4 red[3][8][64];
+// Forward mixing.  A work-group owns G whole samples of one degree and a slice of the channels.
+// Per stage it streams kFwdKC channels of every sample (one contiguous run each) through LDS
+// with 16-byte lane-contiguous loads, double buffered; wave w owns complex columns
+// 32w .. 32w+31 of the G*M columns and reads its operands from LDS in matrix-core order.  The
+// weights come packed in lane order straight from L2, one stage ahead.
+constexpr int kFwdKC = 16;       // channels per stage (a multiple of 4)
+constexpr int kFwdRegs = 4;      // float4 registers per thread and stage: 4 x 256 x 2 = 2048 complex
+
+__global__ void __launch_bounds__(kThreads, 4)
+wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
+                   const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO,
+                   int stage_cap) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float2* lds = reinterpret_cast<float2*>(smem);                // [2][stage_cap]
     const WmmFwdUnit u = units[blockIdx.x];
     const WmmDeg d = degs[u.deg];
-    switch (d.NC) {
-        case 1: wmm_forward_body<1>(FF, Wp, out, d, u, B, nFF, nO, red); break;
-        case 2: wmm_forward_body<2>(FF, Wp, out, d, u, B, nFF, nO, red); break;
-        default: wmm_forward_body<3>(FF, Wp, out, d, u, B, nFF, nO, red); break;
+    const int b0 = blockIdx.y * d.G;
+    if (b0 >= B) return;                                          // uniform for the whole group
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int nb = min(d.G, B - b0);
+    const int i = lane & 15, kk = lane >> 4;
+    const int M = d.M;
+    const int ncols = nb * M;
+    const bool wave_on = w < d.NC;
+    const size_t total = (size_t)B * nFF;
+    const int n4max = (kFwdKC * M + 2) >> 1;                      // float4 slots of one sample's run
+    const int nslots = nb * n4max;
+
+    // the lane's two complex columns: sample, m, LDS offset of channel 0 of the stage
+    bool ok[2];
+    int col_b[2], col_m[2], lofs[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int q = w * 32 + 2 * i + h;
+        ok[h] = wave_on && q < ncols;
+        col_b[h] = ok[h] ? q / M : 0;
+        col_m[h] = ok[h] ? q - col_b[h] * M : 0;
+        const size_t soff = (size_t)(b0 + col_b[h]) * nFF + d.cumFF;   // parity is the same for every stage
+        lofs[h] = col_b[h] * 2 * n4max + (int)(soff & 1) + col_m[h];
+    }
+
+    float4 pre[kFwdRegs];
+    auto fetch = [&](int k0) {
+        const int n = min(kFwdKC, u.k_end - k0) * M;
+#pragma unroll
+        for (int r = 0; r < kFwdRegs; ++r) {
+            const int id = tid + r * kThreads;
+            pre[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (id < nslots) {
+                const int j = id / n4max, idx = id - j * n4max;
+                const size_t off = (size_t)(b0 + j) * nFF + d.cumFF + (size_t)k0 * M;
+                const size_t first = off & ~(size_t)1;
+                const int n4 = (n + (int)(off & 1) + 1) >> 1;
+                if (idx < n4) {
+                    if (first + 2 * (size_t)idx + 1 < total) {
+                        pre[r] = reinterpret_cast<const float4*>(FF + first)[idx];
+                    } else {
+                        const float2 z = FF[first + 2 * (size_t)idx];
+                        pre[r] = make_float4(z.x, z.y, 0.f, 0.f);
+                    }
+                }
+            }
+        }
+    };
+    auto commit = [&](float2* buf) {
+        float4* dst = reinterpret_cast<float4*>(buf);
+#pragma unroll
+        for (int r = 0; r < kFwdRegs; ++r) {
+            const int id = tid + r * kThreads;
+            if (id < nslots) dst[id] = pre[r];
+        }
+    };
+    constexpr int kSteps = kFwdKC / 4;
+    float an0[kSteps], an1[kSteps];                               // next stage's A operands
+    const size_t ap_step = (size_t)d.nrc * 128;
+    auto fetch_a = [&](int k0) {
+        const float* ap = Wp + ((size_t)(d.wp_base + ((k0 >> 2) * d.nrc + u.rc) * 2)) * 64 + lane;
+        const int steps = (min(kFwdKC, u.k_end - k0) + 3) >> 2;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            an0[s] = an1[s] = 0.f;
+            if (s < steps) {
+                an0[s] = ap[(size_t)s * ap_step];
+                an1[s] = ap[(size_t)s * ap_step + 64];
+            }
+        }
+    };
+
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        acc[1][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    if (u.k_begin < u.k_end) {
+        fetch(u.k_begin);
+        if (wave_on) fetch_a(u.k_begin);
+    }
+    int buf = 0;
+    for (int k0 = u.k_begin; k0 < u.k_end; k0 += kFwdKC, buf ^= 1) {
+        float2* cur = lds + (size_t)buf * stage_cap;
+        commit(cur);
+        float a0[kSteps], a1[kSteps];
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            a0[s] = an0[s];
+            a1[s] = an1[s];
+        }
+        __syncthreads();
+        if (k0 + kFwdKC < u.k_end) {
+            fetch(k0 + kFwdKC);
+            if (wave_on) fetch_a(k0 + kFwdKC);
+        }
+        if (wave_on) {
+            const int klen = min(kFwdKC, u.k_end - k0);
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) {
+                const int kl = 4 * s + kk;
+                float2 v0 = make_float2(0.f, 0.f), v1 = v0;
+                if (kl < klen) {
+                    if (ok[0]) v0 = cur[lofs[0] + kl * M];
+                    if (ok[1]) v1 = cur[lofs[1] + kl * M];
+                }
+                acc[0][0] = mfma4(a0[s], v0.x, acc[0][0]);
+                acc[0][1] = mfma4(a0[s], v0.y, acc[0][1]);
+                acc[0][2] = mfma4(a0[s], v1.x, acc[0][2]);
+                acc[0][3] = mfma4(a0[s], v1.y, acc[0][3]);
+                acc[1][0] = mfma4(a1[s], v0.x, acc[1][0]);
+                acc[1][1] = mfma4(a1[s], v0.y, acc[1][1]);
+                acc[1][2] = mfma4(a1[s], v1.x, acc[1][2]);
+                acc[1][3] = mfma4(a1[s], v1.y, acc[1][3]);
+            }
+        }
+    }
+    mfma_drain();
+    // complex outputs: the re / im columns of a complex column sit in the same lane
+    float2* dst = out + (size_t)u.slice * B * nO;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        if (!ok[h]) continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int to = u.rc * 16 + 4 * kk + v;
+            if (to < d.tO) {
+                const float re = acc[0][2 * h][v] - acc[1][2 * h + 1][v];
+                const float im = acc[0][2 * h + 1][v] + acc[1][2 * h][v];
+                dst[(size_t)(b0 + col_b[h]) * nO + d.cumO + to * M + col_m[h]] = make_float2(re, im);
+            }
+        }
     }
 }
 
@@ -323,48 +409,81 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
 // --------------------------------------------------------------------------- grad W (MFMA)
 // Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples (blockIdx.y)
 // into part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
+constexpr int kGwFFRegs = 4;    // 4 x 256 x 16 B = 16 KB of FF per sample and work-group
+constexpr int kGwGORegs = 3;    // 3 x 256 x 16 B = 12 KB of gO rows (16 rows of up to 95 complex)
+
+// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples (blockIdx.y)
+// into part[chunk][nW].  Per sample the group's FF rows (nc channels x M, one contiguous run) and
+// the 16 gO rows are streamed through LDS with 16-byte lane-contiguous loads, double buffered;
+// each wave then reads its 16 channel rows in matrix-core operand order.
 __global__ void __launch_bounds__(kThreads)
 wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, float2* __restrict__ part,
                  const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
-                 int samples_per_chunk, int nFF, int nO, int nW) {
+                 int samples_per_chunk, int nFF, int nO, int nW, int ff_cap, int go_cap) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float2* ffbuf = reinterpret_cast<float2*>(smem);              // [2][ff_cap]
+    float2* gobuf = ffbuf + 2 * ff_cap;                           // [2][go_cap]
     const WmmChanUnit u = units[blockIdx.x];
     const WmmDeg d = degs[u.deg];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int i = lane & 15, kk = lane >> 4;
     const int M = d.M;
-    const int c = u.c0 + 16 * w + i;          // B operand: mid channel of this lane
-    const bool cok = c < d.K && (16 * w + i) < u.nc;
-    const int to_a = u.rc * 16 + i;           // A operand: output channel of this lane
+    const bool wave_on = 16 * w < u.nc;
+    const int c = u.c0 + 16 * w + i;
+    const bool cok = wave_on && c < d.K && (16 * w + i) < u.nc;
+    const int to_a = u.rc * 16 + i;
     const bool tok = to_a < d.tO;
+    const int go_rows = min(16, d.tO - u.rc * 16);
     const int nblk = (M + 7) >> 3;
-    const size_t f_row = (size_t)d.cumFF + (size_t)(cok ? c : 0) * M;
-    const size_t g_row = (size_t)d.cumO + (size_t)(tok ? to_a : 0) * M;
-
-    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const int n_ff = u.nc * M, n_go = go_rows * M;
+    const size_t tot_ff = (size_t)B * nFF, tot_go = (size_t)B * nO;
     const int b_begin = blockIdx.y * samples_per_chunk;
     const int b_end = min(B, b_begin + samples_per_chunk);
-    for (int b = b_begin; b < b_end; ++b) {
-        const float2* frow = FF + (size_t)b * nFF + f_row;
-        const float2* grow = gO + (size_t)b * nO + g_row;
-        for (int blk = 0; blk < nblk; ++blk) {
-            const int p0 = blk * 8 + kk * 2;
-            float2 f0 = make_float2(0.f, 0.f), f1 = f0, g0 = f0, g1 = f0;
-            if (p0 < M) {
-                if (cok) f0 = frow[p0];
-                if (tok) g0 = grow[p0];
+
+    Run16<kGwFFRegs> pf;
+    Run16<kGwGORegs> pg;
+    auto ff_off = [&](int b) { return (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M; };
+    auto go_off = [&](int b) { return (size_t)b * nO + d.cumO + (size_t)u.rc * 16 * M; };
+    if (b_begin < b_end) {
+        pf.fetch(FF, ff_off(b_begin), n_ff, tot_ff, tid, kThreads);
+        pg.fetch(gO, go_off(b_begin), n_go, tot_go, tid, kThreads);
+    }
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    int buf = 0;
+    for (int b = b_begin; b < b_end; ++b, buf ^= 1) {
+        float2* ffl = ffbuf + buf * ff_cap;
+        float2* gol = gobuf + buf * go_cap;
+        const size_t fo = ff_off(b), go_ = go_off(b);
+        pf.commit(ffl, fo, n_ff, tid, kThreads);
+        pg.commit(gol, go_, n_go, tid, kThreads);
+        __syncthreads();
+        if (b + 1 < b_end) {
+            pf.fetch(FF, ff_off(b + 1), n_ff, tot_ff, tid, kThreads);
+            pg.fetch(gO, go_off(b + 1), n_go, tot_go, tid, kThreads);
+        }
+        if (wave_on) {
+            const float2* frow = ffl + (fo & 1) + (cok ? (16 * w + i) : 0) * M;
+            const float2* grow = gol + (go_ & 1) + (tok ? i : 0) * M;
+            for (int blk = 0; blk < nblk; ++blk) {
+                const int p0 = blk * 8 + kk * 2;
+                float2 f0 = make_float2(0.f, 0.f), f1 = f0, g0 = f0, g1 = f0;
+                if (p0 < M) {
+                    if (cok) f0 = frow[p0];
+                    if (tok) g0 = grow[p0];
+                }
+                if (p0 + 1 < M) {
+                    if (cok) f1 = frow[p0 + 1];
+                    if (tok) g1 = grow[p0 + 1];
+                }
+                acc0 = mfma4(g0.x, f0.x, acc0);
+                acc0 = mfma4(g0.y, f0.y, acc0);
+                acc0 = mfma4(g1.x, f1.x, acc0);
+                acc0 = mfma4(g1.y, f1.y, acc0);
+                acc1 = mfma4(g0.y, f0.x, acc1);
+                acc1 = mfma4(-g0.x, f0.y, acc1);
+                acc1 = mfma4(g1.y, f1.x, acc1);
+                acc1 = mfma4(-g1.x, f1.y, acc1);
             }
-            if (p0 + 1 < M) {
-                if (cok) f1 = frow[p0 + 1];
-                if (tok) g1 = grow[p0 + 1];
-            }
-            acc0 = mfma4(g0.x, f0.x, acc0);
-            acc0 = mfma4(g0.y, f0.y, acc0);
-            acc0 = mfma4(g1.x, f1.x, acc0);
-            acc0 = mfma4(g1.y, f1.y, acc0);
-            acc1 = mfma4(g0.y, f0.x, acc1);
-            acc1 = mfma4(-g0.x, f0.y, acc1);
-            acc1 = mfma4(g1.y, f1.x, acc1);
-            acc1 = mfma4(-g1.x, f1.y, acc1);
         }
     }
     mfma_drain();
@@ -433,6 +552,114 @@ wmm_gradff_kernel(const float2* __restrict__ gO, const float2* __restrict__ WT, 
     }
 }
 
+// ---- grad FF on the matrix cores -----------------------------------------------------------
+// gFF[b, c, (m, re/im)] = sum over k = (to, re/im) of A[c][k] * Bop[k][(m, re/im)] with
+//   A[c][(to,0)] = W_re[to][c]/div[c], A[c][(to,1)] = W_im[to][c]/div[c]        (packed once per call)
+//   Bop[(to,0)][(m,0)] = gO_re, Bop[(to,1)][(m,0)] = gO_im, Bop[(to,0)][(m,1)] = gO_im, Bop[(to,1)][(m,1)] = -gO_re
+// A wave keeps the A operand of its 16 channels in registers and walks over the samples of its
+// group; a 16-channel x 16-column result tile is stored as four 64-byte row segments.
+__global__ void __launch_bounds__(256)
+pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                     const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Ap, int total_blocks) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int blk = idx >> 6, lane = idx & 63;
+    if (blk >= total_blocks) return;
+    int di = 0;
+    while (di + 1 < ndeg && degs[di + 1].ap_base <= blk) ++di;
+    const WmmDeg d = degs[di];
+    const int rel = blk - d.ap_base;             // ctile * nks_b + ks
+    const int ks = rel % d.nks_b, ctile = rel / d.nks_b;
+    const int i = lane & 15, kk = lane >> 4;
+    const int c = ctile * 16 + i, k = 4 * ks + kk;
+    const int to = k >> 1, sel = k & 1;
+    float v = 0.f;
+    if (c < d.K && to < d.tO) {
+        const float2 w = W[d.cumW + (size_t)to * d.K + c];
+        v = sel ? w.y : w.x;
+        if (stds) v /= fmaxf(eps, stds[d.cumT + c]);
+    }
+    Ap[idx] = v;
+}
+
+constexpr int kGffGORegs = 3;   // float4 registers per thread for the gO rows of one sample (t_O <= 16 rows)
+
+__global__ void __launch_bounds__(kThreads)
+wmm_gradff_mfma_kernel(const float2* __restrict__ gO, const float* __restrict__ Ap, float2* __restrict__ gFF,
+                       const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
+                       int samples_per_group, int nFF, int nO, int out_cap, int go_cap) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* outbuf = reinterpret_cast<float*>(smem);                          // [2][out_cap] real entries
+    float2* gobuf = reinterpret_cast<float2*>(outbuf + 2 * (size_t)out_cap);  // [2][go_cap]
+    const WmmChanUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const bool wave_on = 16 * w < u.nc;
+    const int i = lane & 15, kk = lane >> 4;
+    const int M = d.M, tO = d.tO, nks = d.nks_b;
+    const int ctile = (u.c0 >> 4) + w;
+    float a[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+        a[ks] = (wave_on && ks < nks) ? Ap[((size_t)d.ap_base + (size_t)ctile * nks + ks) * 64 + lane] : 0.f;
+    const int to_lane = kk >> 1, sel = kk & 1;   // k = 4*ks + kk  ->  to = 2*ks + to_lane, re/im = sel
+    const int nct = (2 * M + 15) >> 4;
+    const int row0 = 16 * w + 4 * kk;            // D rows of this lane inside the group's tile
+    const int n_go = tO * M, n_out = u.nc * M;   // complex entries of the gO rows / of the output run
+    const size_t tot_go = (size_t)B * nO;
+    const int b_begin = blockIdx.y * samples_per_group, b_end = min(B, b_begin + samples_per_group);
+    auto go_off = [&](int b) { return (size_t)b * nO + d.cumO; };
+
+    Run16<kGffGORegs> pg;
+    if (b_begin < b_end) pg.fetch(gO, go_off(b_begin), n_go, tot_go, tid, kThreads);
+    int buf = 0;
+    for (int b = b_begin; b < b_end; ++b, buf ^= 1) {
+        float* ol = outbuf + (size_t)buf * out_cap;
+        float2* gl = gobuf + (size_t)buf * go_cap;
+        const size_t go_ = go_off(b);
+        pg.commit(gl, go_, n_go, tid, kThreads);
+        __syncthreads();                          // gO rows of sample b visible; tile buffer `buf` is free again
+        if (b + 1 < b_end) pg.fetch(gO, go_off(b + 1), n_go, tot_go, tid, kThreads);
+        if (wave_on) {
+            const float2* g = gl + (go_ & 1);
+            for (int ct = 0; ct < nct; ++ct) {
+                const int col = ct * 16 + i;
+                const int m = col >> 1, r = col & 1;
+                const bool cok = m < M;
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) {
+                    if (ks < nks) {
+                        float bv = 0.f;
+                        const int to = 2 * ks + to_lane;
+                        if (cok && to < tO) {
+                            const float2 z = g[to * M + m];
+                            bv = (r == sel) ? (r ? -z.x : z.x) : z.y;
+                        }
+                        acc = mfma4(a[ks], bv, acc);
+                    }
+                }
+                mfma_drain();
+                if (cok) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) ol[(size_t)(row0 + v) * 2 * M + col] = acc[v];
+                }
+            }
+        }
+        __syncthreads();                          // the tile of sample b is complete
+        // stream the tile out: one contiguous run of n_out complex numbers
+        float2* dst = gFF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M;
+        const float2* src = reinterpret_cast<const float2*>(ol);
+        const int head = (int)(((size_t)b * nFF + d.cumFF + (size_t)u.c0 * M) & 1);   // unaligned first entry
+        if (head && tid == 0 && n_out > 0) dst[0] = src[0];
+        const int n4 = (n_out - head) >> 1;
+        for (int idx = tid; idx < n4; idx += kThreads) {
+            const float2 z0 = src[head + 2 * idx], z1 = src[head + 2 * idx + 1];
+            *reinterpret_cast<float4*>(dst + head + 2 * idx) = make_float4(z0.x, z0.y, z1.x, z1.y);
+        }
+        if (((n_out - head) & 1) && tid == 0) dst[n_out - 1] = src[n_out - 1];
+    }
+}
+
 __global__ void __launch_bounds__(256) fill_zero_kernel(float* p, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0.f;
@@ -466,7 +693,8 @@ using namespace cgnet;
 
 static void free_plan(cgnet_wmm_plan* plan) {
     if (!plan) return;
-    void* ptrs[] = {plan->d_degs, plan->d_fwd_units, plan->d_gw_units, plan->d_gff_units, plan->d_stat_units, plan->d_cumO};
+    void* ptrs[] = {plan->d_degs, plan->d_fwd_units, plan->d_gw_units, plan->d_gw_units_rc0, plan->d_gff_units,
+                    plan->d_stat_units, plan->d_cumO};
     for (void* q : ptrs)
         if (q) (void)hipFree(q);
     delete plan;
@@ -505,8 +733,12 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         }
         d.G = bestG;
         d.NC = bestNC;
-        // k-slices of about 1024 channels (multiples of 4)
-        d.S = std::max(1, (K + 1023) / 1024);
+        // k-slices of about 768 channels (multiples of 4)
+        d.S = std::max(1, (K + 767) / 768);
+        d.nks_b = std::max(1, (2 * tO + 3) / 4);
+        d.ap_base = p->ap_blocks;
+        p->ap_blocks += ((K + 15) / 16) * d.nks_b;
+        if (tO > 16) p->gff_mfma = false;
         p->degs.push_back(d);
         cFF += (long long)K * M;
         cO += (long long)tO * M;
@@ -524,6 +756,7 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         CGNET_REQUIRE(d.NC <= 3, CGNET_ERR_UNSUPPORTED, "degree %d has more than 96 columns per sample", d.l);
         p->maxS = std::max(p->maxS, d.S);
         p->maxG = std::max(p->maxG, d.G);
+        p->fwd_stage_cap = std::max(p->fwd_stage_cap, d.G * 2 * ((kFwdKC * d.M + 2) / 2));
         const int steps = (d.K + 3) / 4;
         const int per = ((steps + d.S - 1) / d.S) * 4;
         for (int rc = 0; rc < d.nrc; ++rc)
@@ -531,8 +764,15 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
                 WmmFwdUnit u{di, rc, s, std::min(d.K, s * per), std::min(d.K, (s + 1) * per)};
                 p->fwd_units.push_back(u);
             }
+        int gw_nc = 64;
+        while (gw_nc > 16 && (size_t)gw_nc * d.M + 2 > (size_t)kGwFFRegs * kThreads * 2) gw_nc /= 2;
         for (int rc = 0; rc < d.nrc; ++rc)
-            for (int c0 = 0; c0 < d.K; c0 += 64) p->gw_units.push_back(WmmChanUnit{di, rc, c0, std::min(64, d.K - c0)});
+            for (int c0 = 0; c0 < d.K; c0 += gw_nc)
+                p->gw_units.push_back(WmmChanUnit{di, rc, c0, std::min(gw_nc, d.K - c0)});
+        p->gff_out_cap = std::max(p->gff_out_cap, (int)align_up((size_t)gw_nc * d.M * 2, 4));
+        p->gff_go_cap = std::max(p->gff_go_cap, (int)align_up((size_t)std::min(d.tO, 16) * d.M + 2, 2));
+        p->gw_ff_cap = std::max(p->gw_ff_cap, (int)align_up((size_t)gw_nc * d.M + 2, 2));
+        p->gw_go_cap = std::max(p->gw_go_cap, (int)align_up((size_t)16 * d.M + 2, 2));
     }
     for (int di = 0; di < ndeg; ++di) {
         const WmmDeg& d = p->degs[di];
@@ -570,6 +810,9 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
     if ((rc = upload(p->degs.data(), sizeof(WmmDeg) * ndeg, (void**)&p->d_degs))) return rc;
     if ((rc = upload(p->fwd_units.data(), sizeof(WmmFwdUnit) * p->fwd_units.size(), (void**)&p->d_fwd_units))) return rc;
     if ((rc = upload(p->gw_units.data(), sizeof(WmmChanUnit) * p->gw_units.size(), (void**)&p->d_gw_units))) return rc;
+    for (const WmmChanUnit& u : p->gw_units)
+        if (u.rc == 0) p->gw_units_rc0.push_back(u);
+    if ((rc = upload(p->gw_units_rc0.data(), sizeof(WmmChanUnit) * p->gw_units_rc0.size(), (void**)&p->d_gw_units_rc0))) return rc;
     if ((rc = upload(p->gff_units.data(), sizeof(WmmChanUnit) * p->gff_units.size(), (void**)&p->d_gff_units))) return rc;
     if ((rc = upload(p->stat_units.data(), sizeof(WmmChanUnit) * p->stat_units.size(), (void**)&p->d_stat_units))) return rc;
     if ((rc = upload(cumO_S.data(), sizeof(int) * cumO_S.size(), (void**)&p->d_cumO))) return rc;
@@ -664,8 +907,10 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     for (const WmmDeg& d : plan->degs)
         if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + d.G - 1) / d.G);
     CGNET_REQUIRE(ygroups <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d too large", B);
-    CGNET_LAUNCH(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads), 0, s,
-                       d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO);
+    CGNET_REQUIRE(((uintptr_t)d_FF & 15) == 0, CGNET_ERR_ARG, "d_FF must be 16-byte aligned");
+    CGNET_LAUNCH(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads),
+                 sizeof(float2) * 2 * (size_t)plan->fwd_stage_cap, s, (const float2*)d_FF, Wp, out, plan->d_degs,
+                 plan->d_fwd_units, B, plan->nFF, plan->nO, plan->fwd_stage_cap);
     CGNET_HIP(hipGetLastError());
     if (plan->maxS > 1) {
         const size_t n = (size_t)plan->nO * B;
@@ -677,11 +922,14 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
 }
 
 static int gradw_chunks(int B) { return (B + kGradWChunk - 1) / kGradWChunk; }
+static size_t gff_operand_bytes(const cgnet_wmm_plan* plan) {
+    return plan->gff_mfma ? sizeof(float) * 64 * (size_t)plan->ap_blocks : sizeof(float) * 2 * (size_t)plan->nW;
+}
 
 extern "C" size_t cgnet_FN_WMM_backward_workspace(const cgnet_wmm_plan* plan, int B) {
     if (!plan || B <= 0) return 0;
-    // [conj(W)/div, channel-major] [raw weight-gradient sums per chunk of samples]
-    return align_up(sizeof(float) * 2 * (size_t)plan->nW, 256) +
+    // [operand of the FF-gradient kernel] [raw weight-gradient sums per chunk of samples]
+    return align_up(gff_operand_bytes(plan), 256) +
            align_up(sizeof(float) * 2 * (size_t)plan->nW * gradw_chunks(B), 256);
 }
 
@@ -693,13 +941,15 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
     CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
     const bool bn = flags & CGNET_FN_BATCHNORM;
     CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    CGNET_REQUIRE(((uintptr_t)d_gO & 15) == 0 && ((uintptr_t)d_FF & 15) == 0 && ((uintptr_t)d_gFF & 15) == 0,
+                  CGNET_ERR_ARG, "d_gO, d_FF and d_gFF must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const int ndeg = (int)plan->degs.size();
     const size_t need = cgnet_FN_WMM_backward_workspace(plan, B);
     CGNET_REQUIRE(B == 0 || (d_workspace && workspace_bytes >= need), CGNET_ERR_WORKSPACE,
                   "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     float2* WT = (float2*)d_workspace;
-    float2* gw_part = (float2*)((char*)d_workspace + align_up(sizeof(float) * 2 * (size_t)plan->nW, 256));
+    float2* gw_part = (float2*)((char*)d_workspace + align_up(gff_operand_bytes(plan), 256));
     if (d_gW && plan->nW > 0) {
         if (B == 0 || plan->nO == 0) {
             const size_t n = (size_t)2 * plan->nW;
@@ -708,9 +958,10 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         } else {
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
             const int nchunks = gradw_chunks(B);
-            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), 0, s,
+            const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
+            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), lds, s,
                                (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
-                               kGradWChunk, plan->nFF, plan->nO, plan->nW);
+                               kGradWChunk, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
             CGNET_HIP(hipGetLastError());
             CGNET_LAUNCH(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)gw_part, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg,
@@ -722,15 +973,30 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
         CGNET_REQUIRE(d_W, CGNET_ERR_ARG, "d_W is NULL");
         CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
-        if (plan->nW > 0) {
-            CGNET_LAUNCH(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
-                               (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
+        if (plan->gff_mfma && plan->nW > 0 && plan->nO > 0) {
+            float* Ap = (float*)d_workspace;
+            const int total = plan->ap_blocks * 64;
+            CGNET_LAUNCH(pack_w_gradff_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
+                         bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Ap, plan->ap_blocks);
+            CGNET_HIP(hipGetLastError());
+            const int groups = std::max(1, std::min(B, 8));
+            const int spg = (B + groups - 1) / groups;
+            const size_t lds = 2 * (sizeof(float) * (size_t)plan->gff_out_cap + sizeof(float2) * (size_t)plan->gff_go_cap);
+            CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)plan->gw_units_rc0.size(), (B + spg - 1) / spg),
+                         dim3(kThreads), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
+                         plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, plan->gff_out_cap, plan->gff_go_cap);
+            CGNET_HIP(hipGetLastError());
+        } else {
+            if (plan->nW > 0) {
+                CGNET_LAUNCH(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
+                             (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
+                CGNET_HIP(hipGetLastError());
+            }
+            CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
+                         plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
+                         plan->d_gff_units, plan->nFF, plan->nO);
             CGNET_HIP(hipGetLastError());
         }
-        CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
-                           plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
-                           plan->d_gff_units, plan->nFF, plan->nO);
-        CGNET_HIP(hipGetLastError());
     }
     return CGNET_OK;
 }
