@@ -476,13 +476,14 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 
 // ---- register-resident backward ------------------------------------------------------------
 struct BwdGeom { int l, l1, l2, rows, tau2; };
+constexpr int kBwdMaxTI = 4;   // output channels per thread
 
 // Adds one task's contribution to the calling thread's accumulators.  Same arithmetic and item
 // layout as bwd_phase, one item per thread (rtid = thread index inside its role), no reduction.
 template <int SLOT, int TI, int RW>
 __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restrict__ cgp,
                                           const float2* __restrict__ g, const float2* __restrict__ fr,
-                                          int rtid, float (&ax)[4][2], float (&ay)[4][2]) {
+                                          int rtid, float (&ax)[kBwdMaxTI][2], float (&ay)[kBwdMaxTI][2]) {
     const int l = q.l, l1 = q.l1, l2 = q.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int Mp = M + kPadLo + kPadHi;
@@ -506,7 +507,7 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     for (int i = 0; i < TI; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
     const int col0 = min(mo0, M2 - 1), col1 = min(mo0 + 1, M2 - 1);
     for (int r = lane_r; r < n_r; r += RW) {
-        const float2* frow = fr + r * M_r;
+        const float2* frow = fr + r * (M_r + 1);      // rows carry one trailing zero
         const float2* gb = g + r * g_sr + (kPadLo + mo0 - d);
         const float* cb = cgp + (kPadLo + mo0 - d) * M2;
         float2 e0[TI], e1[TI];
@@ -535,12 +536,12 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
 #pragma unroll
             for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir + 2];
             {
+                // past the valid range either the fragment (padded row), the table row (padded) or
+                // the tile entry (padded m axis) is zero, so no masking is needed
                 const int ir1 = ir + 1;
-                const int irc = min(ir1, M_r - 1);
-                float2 f = frow[irc];
-                if (ir1 > ir_hi) f = make_float2(0.f, 0.f);
-                const float c0 = (SLOT == 1) ? cb[ir1 * M2 + irc] : cb[ir1 * M2 + col0];
-                const float c1 = (SLOT == 1) ? cb[(ir1 + 1) * M2 + irc] : cb[(ir1 + 1) * M2 + col1];
+                const float2 f = frow[ir1];
+                const float c0 = (SLOT == 1) ? cb[ir1 * M2 + ir1] : cb[ir1 * M2 + col0];
+                const float c1 = (SLOT == 1) ? cb[(ir1 + 1) * M2 + ir1] : cb[(ir1 + 1) * M2 + col1];
                 const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
 #pragma unroll
                 for (int i = 0; i < TI; ++i) {
@@ -561,8 +562,8 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
 // Adds up the RW lanes of every item (all lanes of the wave take part) and stores the slab
 // dst[n_o][M_o]; every element of the slab has exactly one owner.  Clears the accumulators.
 template <int TI, int RW>
-__device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax)[4][2], float (&ay)[4][2],
-                                          float2* __restrict__ dst) {
+__device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax)[kBwdMaxTI][2],
+                                          float (&ay)[kBwdMaxTI][2], float2* __restrict__ dst) {
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
         ax[i][0] = row_sum<RW>(ax[i][0]);
@@ -588,7 +589,7 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+    for (int i = 0; i < kBwdMaxTI; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
 }
 
 #define CGNET_BWD_SWITCH(TI_, RW_, CALL)                                         \
@@ -651,12 +652,15 @@ __device__ __forceinline__ void bwd_prefetch(BwdPrefetch& pf, const BwdUTask& t,
         if (e < ncg && x >= 0 && x < M * M2) pf.cg[k] = CG[t.cg_off + x];
     }
     if (t.first_of_l2) {
-        const int n2 = t.tau2 * M2;
+        const int n2p = t.tau2 * (M2 + 1);            // rows padded by one zero
+        const float inv2 = 1.0f / (float)(M2 + 1);
 #pragma unroll
         for (int k = 0; k < kPreF; ++k) {
             const int e = tid + k * kThreads;
+            const int row = (int)(((float)e + 0.5f) * inv2);
+            const int x = e - row * (M2 + 1);
             pf.f2[k] = make_float2(0.f, 0.f);
-            if (e < n2) pf.f2[k] = Fb[t.offF2 + e];
+            if (e < n2p && x < M2) pf.f2[k] = Fb[t.offF2 + row * M2 + x];
         }
     }
 }
@@ -669,7 +673,8 @@ __device__ __forceinline__ void bwd_commit(const BwdPrefetch& pf, const BwdUTask
                                            float2* __restrict__ f2, float* __restrict__ cgp, float2* __restrict__ g) {
     const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
     const int Mp = M + kPadLo + kPadHi;
-    const int ntile = rows * t.tau2 * Mp, ncg = Mp * M2, n2 = t.tau2 * M2;
+    const int ntile = rows * t.tau2 * Mp, ncg = Mp * M2, n2p = t.tau2 * (M2 + 1);
+    if (tid == 0) cgp[ncg] = 0.f;                     // one entry past the table may be read (times zero)
 #pragma unroll
     for (int k = 0; k < kPreTile; ++k) {
         const int e = tid + k * kThreads;
@@ -684,9 +689,14 @@ __device__ __forceinline__ void bwd_commit(const BwdPrefetch& pf, const BwdUTask
 #pragma unroll
         for (int k = 0; k < kPreF; ++k) {
             const int e = tid + k * kThreads;
-            if (e < n2) f2[e] = pf.f2[k];
+            if (e < n2p) f2[e] = pf.f2[k];
         }
-        for (int e = tid + kPreF * kThreads; e < n2; e += kThreads) f2[e] = Fb[t.offF2 + e];
+        const float inv2 = 1.0f / (float)(M2 + 1);
+        for (int e = tid + kPreF * kThreads; e < n2p; e += kThreads) {
+            const int row = (int)(((float)e + 0.5f) * inv2);
+            const int x = e - row * (M2 + 1);
+            f2[e] = x < M2 ? Fb[t.offF2 + row * M2 + x] : make_float2(0.f, 0.f);
+        }
     }
     if (ntile > kPreTile * kThreads) {
         const float inv = 1.0f / (float)Mp;
@@ -721,8 +731,8 @@ __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int
                                           BwdUTask& t, BwdUTask& cur, float*& cgp, float2*& g) {
     const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
     const int Mp = M + kPadLo + kPadHi;
-    cgp = reinterpret_cast<float*>(c.f2 + t.tau2 * M2);
-    g = reinterpret_cast<float2*>(cgp + ((Mp * M2 + 1) & ~1));
+    cgp = reinterpret_cast<float*>(c.f2 + t.tau2 * (M2 + 1));
+    g = reinterpret_cast<float2*>(cgp + ((Mp * M2 + 2) & ~1));
     __syncthreads();                                 // the previous tile (and f2) are no longer read
     bwd_commit(pf, t, u.rows, c.Gb, c.Fb, c.CG, c.tid, c.f2, cgp, g);
     __syncthreads();
@@ -737,9 +747,9 @@ __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int
 template <int TI, int RW>
 __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
                                                 float2* __restrict__ dst) {
-    float ax[4][2], ay[4][2], tx[4][2], ty[4][2];
+    float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kBwdMaxTI; ++i) {
         ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
         tx[i][0] = tx[i][1] = ty[i][0] = ty[i][1] = 0.f;
     }
@@ -753,7 +763,7 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TI; ++i)
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
                     tx[i][k] += ax[i][k];
@@ -768,9 +778,9 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
 // Waves of role B: gradient of slot 2, kept in registers across the tasks that share l2.
 __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
                                                 float2* __restrict__ part2_b) {
-    float ax[4][2], ay[4][2];
+    float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+    for (int i = 0; i < kBwdMaxTI; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
     for (int ti = u.task_begin; ti < u.task_end; ++ti) {
         BwdUTask cur;
         float* cgp;
@@ -806,14 +816,21 @@ cg_backward_unit_kernel(const float2* __restrict__ F, const float2* __restrict__
     c.CG = CG;
     c.tasks = tasks;
     c.f1 = reinterpret_cast<float2*>(smem);
-    c.f2 = c.f1 + u.rows * M1;
+    c.f2 = c.f1 + u.rows * (M1 + 1);
     c.tid = tid;
     c.rtid = roleA ? tid : tid - 64 * u.nA;
 
     BwdPrefetch pf;
     const BwdUTask t0 = tasks[u.task_begin];
     bwd_prefetch(pf, t0, u.rows, c.Gb, c.Fb, CG, tid);
-    for (int e = tid; e < u.rows * M1; e += kThreads) c.f1[e] = c.Fb[u.offF1 + e];
+    {
+        const float inv1 = 1.0f / (float)(M1 + 1);
+        for (int e = tid; e < u.rows * (M1 + 1); e += kThreads) {
+            const int row = (int)(((float)e + 0.5f) * inv1);
+            const int x = e - row * (M1 + 1);
+            c.f1[e] = x < M1 ? c.Fb[u.offF1 + row * M1 + x] : make_float2(0.f, 0.f);
+        }
+    }
 
     // The two roles run the same sequence of barriers (two per task) from different code paths.
     if (roleA) {
@@ -1115,7 +1132,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     for (int k = 0; k < nt && feasible; ++k) {
                         const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
                         double bc = -1;
-                        for (int ti = 1; ti <= 4; ++ti)
+                        for (int ti = 1; ti <= kBwdMaxTI; ++ti)
                             for (int rw = 1; rw <= 16; rw *= 2) {
                                 if (rw > 1 && rw / 2 >= rows_c) continue;
                                 const int items = ((tau2 + ti - 1) / ti) * ((M2 + 1) / 2);
@@ -1129,7 +1146,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     if (!feasible) continue;
                     int max_tau2 = 1;
                     for (int i : tri) max_tau2 = std::max(max_tau2, h_t_F[tl2[i]]);
-                    for (int ti = 1; ti <= 4; ++ti)
+                    for (int ti = 1; ti <= kBwdMaxTI; ++ti)
                         for (int rw = 1; rw <= 16; rw *= 2) {
                             if (rw > 1 && rw / 2 >= max_tau2) continue;
                             const int items = ((rows_c + ti - 1) / ti) * ((M1 + 1) / 2);
@@ -1177,11 +1194,11 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     }
                     t.TI = best.bTI[k]; t.RW = best.bRW[k];
                     p->bwd_utasks.push_back(t);
-                    task_lds = std::max(task_lds, (size_t)8 * t.tau2 * M2 + 4 * (size_t)((Mp * M2 + 1) & ~1) +
+                    task_lds = std::max(task_lds, (size_t)8 * t.tau2 * (M2 + 1) + 4 * (size_t)((Mp * M2 + 2) & ~1) +
                                                       (size_t)8 * u.rows * t.tau2 * Mp);
                 }
                 u.task_end = (int)p->bwd_utasks.size();
-                lds_max = std::max(lds_max, (size_t)8 * u.rows * M1 + task_lds);
+                lds_max = std::max(lds_max, (size_t)8 * u.rows * (M1 + 1) + task_lds);
                 p->bwd_units.push_back(u);
                 unit_cost.push_back(best.total);
             }
