@@ -129,7 +129,9 @@ def main():
         "cg_forward_kernel": 8 * bsz * (n_f + n_ff),
         "wmm_forward_kernel": 8 * (bsz * n_ff + n_w + bsz * n_o) + 4 * sum_t,
         "wmm_gradw_kernel": 8 * (bsz * n_ff + bsz * n_o + n_w),
+        "wmm_gradff_mfma_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
         "wmm_gradff_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
+        "cg_backward_unit_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
