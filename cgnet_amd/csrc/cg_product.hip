@@ -16,6 +16,7 @@
 // and combines with a fixed DPP tree, so the result does not depend on scheduling.  Groups
 // write partial gradients that a second kernel adds in a fixed order.
 #include <algorithm>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
@@ -43,6 +44,7 @@ struct CgTask {
 struct BwdUnit {
     int l1, rows;
     int offF1;                // complex offset inside a sample's F of the unit's first row
+    int offF1p;               // the same inside a sample's padded fragments (rows of 2*l1+2 entries)
     int task_begin, task_end; // range in the unit-ordered task array (sorted by l2, then l)
     int nA;                   // waves that take slot 1; the other waves of the group take slot 2
     int TI, RW;               // slot-1 tiling: output rows per thread, lanes sharing one output
@@ -52,7 +54,9 @@ struct BwdUTask {
     int l, l2, tau2;
     int offFF;                // complex offset inside a sample's gFF of the tile
     int offF2;                // complex offset inside a sample's F of degree l2
+    int offF2p;               // the same inside a sample's padded fragments
     int cg_off;
+    int cgp_off, cgp_len;     // float offset / length (multiple of 4) of the triple's zero-padded table
     int p2off;                // complex offset inside a sample's slot-2 partial area of this (unit, l2) slab
     int first_of_l2, last_of_l2;
     int TI, RW;               // slot-2 tiling for this run of equal l2
@@ -79,6 +83,10 @@ struct cgnet_cg_plan {
     cgnet::BwdUnit* d_bwd_units = nullptr;
     cgnet::BwdUTask* d_bwd_utasks = nullptr;
     int* d_bwd_combine = nullptr;                // [L+2] cumF | [L+1] own1 | [L+2] list begin | list of slab offsets
+    int* d_bwd_padmeta = nullptr;                // [L+2] cumF | [L+2] cumFp | per triple {cg_off, cgp_off, cgp_len, M, M2}
+    int bwd_nFp = 0;                             // complex entries of one sample's padded fragments
+    int bwd_cgp_len = 0;                         // floats of all padded tables
+    int bwd_f1cap = 0, bwd_f2cap = 0, bwd_cgcap = 0, bwd_tcap = 0;   // LDS bytes of the staged operands
     int bwd_P2 = 0;                              // complex entries of one sample's slot-2 partial area
     size_t bwd_fast_lds = 0;
     int device = 0;
@@ -93,6 +101,7 @@ constexpr int kBwdTileBytes = 16 * 1024;
 constexpr int kMaxTileChannels = 4 * kThreads;   // statistics: at most four channels per thread
 constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
+constexpr size_t kMaxUnitLds = 64 * 1024;       // unit backward: LDS-direct copies address the first 64 KB
 
 __host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
     const size_t M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
@@ -261,7 +270,7 @@ __device__ __forceinline__ float row_sum(float v) {
 
 // Zero padding of the m axis of the staged gFF tile and of the CG table rows: the two m
 // outputs of a thread and the two-step unrolled loop may touch one index below and two above.
-constexpr int kPadLo = 1, kPadHi = 2;
+constexpr int kPadLo = 1, kPadHi = 3;
 
 __host__ __device__ inline size_t bwd_task_lds(const CgTask& t) {
     const size_t M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
@@ -477,22 +486,27 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 // ---- register-resident backward ------------------------------------------------------------
 struct BwdGeom { int l, l1, l2, rows, tau2; };
 constexpr int kBwdMaxTI = 4;   // output channels per thread
+// Zero rows before / after the staged CG table.  The two m outputs of a thread and the two-step
+// unrolled loop touch table rows -1 .. M+1; there the coefficient is zero, so whatever finite
+// value the tile holds at the matching position (the neighbouring channel) does not count.
+constexpr int kTabLo = 1, kTabHi = 2;
 
 // Adds one task's contribution to the calling thread's accumulators.  Same arithmetic and item
 // layout as bwd_phase, one item per thread (rtid = thread index inside its role), no reduction.
+// g: the tile exactly as it lies in gFF ([t1][t2][m], no padding); cgp: the table with kTabLo /
+// kTabHi zero rows; fr: fragment rows of the reduced slot with one trailing zero each.
 template <int SLOT, int TI, int RW>
 __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restrict__ cgp,
                                           const float2* __restrict__ g, const float2* __restrict__ fr,
                                           int rtid, float (&ax)[kBwdMaxTI][2], float (&ay)[kBwdMaxTI][2]) {
     const int l = q.l, l1 = q.l1, l2 = q.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
-    const int Mp = M + kPadLo + kPadHi;
     const int rows = q.rows, tau2 = q.tau2;
     const int n_o = (SLOT == 1) ? rows : tau2;
     const int n_r = (SLOT == 1) ? tau2 : rows;
     const int M_o = (SLOT == 1) ? M1 : M2, M_r = (SLOT == 1) ? M2 : M1;
-    const int g_so = (SLOT == 1) ? tau2 * Mp : Mp;
-    const int g_sr = (SLOT == 1) ? Mp : tau2 * Mp;
+    const int g_so = (SLOT == 1) ? tau2 * M : M;
+    const int g_sr = (SLOT == 1) ? M : tau2 * M;
     const int d = l1 + l2 - l;
     const int item = rtid / RW, lane_r = rtid % RW;
     const int nT = (n_o + TI - 1) / TI;
@@ -508,8 +522,8 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     const int col0 = min(mo0, M2 - 1), col1 = min(mo0 + 1, M2 - 1);
     for (int r = lane_r; r < n_r; r += RW) {
         const float2* frow = fr + r * (M_r + 1);      // rows carry one trailing zero
-        const float2* gb = g + r * g_sr + (kPadLo + mo0 - d);
-        const float* cb = cgp + (kPadLo + mo0 - d) * M2;
+        const float2* gb = g + r * g_sr + (mo0 - d);
+        const float* cb = cgp + (kTabLo + mo0 - d) * M2;
         float2 e0[TI], e1[TI];
 #pragma unroll
         for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir_lo];
@@ -536,8 +550,8 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
 #pragma unroll
             for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir + 2];
             {
-                // past the valid range either the fragment (padded row), the table row (padded) or
-                // the tile entry (padded m axis) is zero, so no masking is needed
+                // past the valid range either the fragment (padded row) or the table row (padded)
+                // is zero, so no masking is needed
                 const int ir1 = ir + 1;
                 const float2 f = frow[ir1];
                 const float c0 = (SLOT == 1) ? cb[ir1 * M2 + ir1] : cb[ir1 * M2 + col0];
@@ -616,136 +630,77 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         default: { CALL(4, 16); } break;                                         \
     }
 
-// Registers that carry the next task's operands while the current task computes.
-constexpr int kPreTile = 8;   // gFF tile elements per thread   (covers 8 * 256 = 2048 complex = 16 KB)
-constexpr int kPreCg = 4;     // CG table entries per thread
-constexpr int kPreF = 2;      // fragment entries per thread
-struct BwdPrefetch {
-    float2 tile[kPreTile];
-    float cg[kPreCg];
-    float2 f2[kPreF];
-};
+// ---- operand staging: global memory -> LDS without passing through registers ----------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
-// Issues the loads of task t (tile with zero padding along m, padded CG table, slab of degree l2).
-__device__ __forceinline__ void bwd_prefetch(BwdPrefetch& pf, const BwdUTask& t, int rows,
-                                             const float2* __restrict__ Gb, const float2* __restrict__ Fb,
-                                             const float* __restrict__ CG, int tid) {
-    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
-    const int Mp = M + kPadLo + kPadHi;
-    const int ntile = rows * t.tau2 * Mp;
-    const float inv = 1.0f / (float)Mp;
-    const float2* src = Gb + t.offFF;
-#pragma unroll
-    for (int k = 0; k < kPreTile; ++k) {
-        const int e = tid + k * kThreads;
-        const int ch = (int)(((float)e + 0.5f) * inv);
-        const int x = e - ch * Mp - kPadLo;
-        pf.tile[k] = make_float2(0.f, 0.f);
-        if (e < ntile && x >= 0 && x < M) pf.tile[k] = src[ch * M + x];
-    }
-    const int ncg = Mp * M2;
-#pragma unroll
-    for (int k = 0; k < kPreCg; ++k) {
-        const int e = tid + k * kThreads;
-        const int x = e - kPadLo * M2;
-        pf.cg[k] = 0.f;
-        if (e < ncg && x >= 0 && x < M * M2) pf.cg[k] = CG[t.cg_off + x];
-    }
-    if (t.first_of_l2) {
-        const int n2p = t.tau2 * (M2 + 1);            // rows padded by one zero
-        const float inv2 = 1.0f / (float)(M2 + 1);
-#pragma unroll
-        for (int k = 0; k < kPreF; ++k) {
-            const int e = tid + k * kThreads;
-            const int row = (int)(((float)e + 0.5f) * inv2);
-            const int x = e - row * (M2 + 1);
-            pf.f2[k] = make_float2(0.f, 0.f);
-            if (e < n2p && x < M2) pf.f2[k] = Fb[t.offF2 + row * M2 + x];
-        }
-    }
+// Starts the copy of `nchunks` 16-byte pieces from `src` (8-byte aligned is enough) to the LDS
+// address `dst` (16-byte aligned).  Lane i of a wave lands 16*i bytes behind the wave's first
+// piece, so consecutive threads fill consecutive pieces.  Nothing may read the destination
+// before dma_wait() and a barrier.
+__device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
+    const char* s = reinterpret_cast<const char*>(src);
+    char* d = reinterpret_cast<char*>(dst);
+    for (int e = tid; e < nchunks; e += kThreads)
+        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
 }
 
-// Writes the prefetched operands of task t into LDS; entries beyond the register window are
-// loaded here directly (large shapes only).
-__device__ __forceinline__ void bwd_commit(const BwdPrefetch& pf, const BwdUTask& t, int rows,
-                                           const float2* __restrict__ Gb, const float2* __restrict__ Fb,
-                                           const float* __restrict__ CG, int tid,
-                                           float2* __restrict__ f2, float* __restrict__ cgp, float2* __restrict__ g) {
-    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
-    const int Mp = M + kPadLo + kPadHi;
-    const int ntile = rows * t.tau2 * Mp, ncg = Mp * M2, n2p = t.tau2 * (M2 + 1);
-    if (tid == 0) cgp[ncg] = 0.f;                     // one entry past the table may be read (times zero)
-#pragma unroll
-    for (int k = 0; k < kPreTile; ++k) {
-        const int e = tid + k * kThreads;
-        if (e < ntile) g[e] = pf.tile[k];
-    }
-#pragma unroll
-    for (int k = 0; k < kPreCg; ++k) {
-        const int e = tid + k * kThreads;
-        if (e < ncg) cgp[e] = pf.cg[k];
-    }
-    if (t.first_of_l2) {
-#pragma unroll
-        for (int k = 0; k < kPreF; ++k) {
-            const int e = tid + k * kThreads;
-            if (e < n2p) f2[e] = pf.f2[k];
-        }
-        const float inv2 = 1.0f / (float)(M2 + 1);
-        for (int e = tid + kPreF * kThreads; e < n2p; e += kThreads) {
-            const int row = (int)(((float)e + 0.5f) * inv2);
-            const int x = e - row * (M2 + 1);
-            f2[e] = x < M2 ? Fb[t.offF2 + row * M2 + x] : make_float2(0.f, 0.f);
-        }
-    }
-    if (ntile > kPreTile * kThreads) {
-        const float inv = 1.0f / (float)Mp;
-        const float2* src = Gb + t.offFF;
-        for (int e = tid + kPreTile * kThreads; e < ntile; e += kThreads) {
-            const int ch = (int)(((float)e + 0.5f) * inv);
-            const int x = e - ch * Mp - kPadLo;
-            float2 v = make_float2(0.f, 0.f);
-            if (x >= 0 && x < M) v = src[ch * M + x];
-            g[e] = v;
-        }
-    }
-    for (int e = tid + kPreCg * kThreads; e < ncg; e += kThreads) {
-        const int x = e - kPadLo * M2;
-        cgp[e] = (x >= 0 && x < M * M2) ? CG[t.cg_off + x] : 0.f;
-    }
+// One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1.
+__device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, int tid) {
+    if (tid < 2)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
 }
+
+// All copies this wave has started have landed (vmcnt == 0).
+__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
 struct BwdCtx {
-    const float2* Fb;          // this sample's fragments
+    const float2* Fp;          // this sample's fragments, rows padded with one zero
     const float2* Gb;          // this sample's gFF
-    const float* CG;
+    const float* CGP;          // zero-padded tables of all triples
     const BwdUTask* tasks;
-    float2* f1;                // LDS: rows x M1 slab of degree l1 (fixed for the unit)
-    float2* f2;                // LDS: slab of the current l2, followed by the CG table and the tile
+    float2* f1;                // LDS: rows x (M1+1) slab of degree l1 (fixed for the unit)
+    char* f2;                  // LDS: two slabs of degree l2 (current run / next run), f2cap bytes each
+    char* cg;                  // LDS: two tables, cgcap bytes each
+    char* tile;                // LDS: two tiles, tcap + 16 bytes each
+    int f2cap, cgcap, tcap;
     int tid, rtid;
 };
 
-// Common per-task prologue of both roles: publish the prefetched operands of task `t` in LDS and
-// start loading the next task's.  Every thread of the group executes the two barriers.
-__device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int ti, BwdPrefetch& pf,
-                                          BwdUTask& t, BwdUTask& cur, float*& cgp, float2*& g) {
+// Starts the copies of task t: tile and table into buffer `par`, the l2 slab (first task of a
+// run only) into slab buffer `f2par`.
+__device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, const BwdUTask& t, int par, int f2par) {
     const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
-    const int Mp = M + kPadLo + kPadHi;
-    cgp = reinterpret_cast<float*>(c.f2 + t.tau2 * (M2 + 1));
-    g = reinterpret_cast<float2*>(cgp + ((Mp * M2 + 2) & ~1));
-    __syncthreads();                                 // the previous tile (and f2) are no longer read
-    bwd_commit(pf, t, u.rows, c.Gb, c.Fb, c.CG, c.tid, c.f2, cgp, g);
-    __syncthreads();
+    const int ntile = u.rows * t.tau2 * M;
+    char* tile = c.tile + par * (c.tcap + 16);
+    dma16(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
+    if (ntile & 1) dma8(c.Gb + t.offFF + (ntile - 1), tile + 8 * (size_t)(ntile - 1), c.tid);
+    dma16(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
+    if (t.first_of_l2) dma16(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
+}
+
+// Per-task prologue of both roles.  On entry `t` is the task whose copies were started one
+// task earlier into buffer `par`; on exit they are visible, `cur` holds that task and the
+// copies of the following task are in flight.  One barrier per task, executed by every thread.
+__device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int ti, BwdUTask& t, BwdUTask& cur,
+                                          int& par, int& f2par, const float*& cgp, const float2*& g,
+                                          const float2*& f2) {
+    dma_wait();
+    __syncthreads();           // copies of every wave landed; nobody still reads the other buffers
     cur = t;
-    if (ti + 1 < u.task_end) {                       // next task's loads fly while this one computes
+    cgp = reinterpret_cast<const float*>(c.cg + par * c.cgcap);
+    g = reinterpret_cast<const float2*>(c.tile + par * (c.tcap + 16));
+    f2 = reinterpret_cast<const float2*>(c.f2 + f2par * c.f2cap);
+    par ^= 1;
+    if (ti + 1 < u.task_end) {
         t = c.tasks[ti + 1];
-        bwd_prefetch(pf, t, u.rows, c.Gb, c.Fb, c.CG, c.tid);
+        if (t.first_of_l2) f2par ^= 1;
+        bwd_issue(c, u, t, par, f2par);
     }
 }
 
 // Waves of role A: gradient of slot 1 (rows of degree l1), kept in registers for the whole unit.
 template <int TI, int RW>
-__device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
+__device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdUTask t,
                                                 float2* __restrict__ dst) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
 #pragma unroll
@@ -753,13 +708,14 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
         tx[i][0] = tx[i][1] = ty[i][0] = ty[i][1] = 0.f;
     }
+    int par = 0, f2par = 0;
     for (int ti = u.task_begin; ti < u.task_end; ++ti) {
         BwdUTask cur;
-        float* cgp;
-        float2* g;
-        bwd_stage(c, u, ti, pf, t, cur, cgp, g);
+        const float* cgp;
+        const float2 *g, *f2;
+        bwd_stage(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
-        bwd_accum<1, TI, RW>(q, cgp, g, c.f2, c.rtid, ax, ay);
+        bwd_accum<1, TI, RW>(q, cgp, g, f2, c.rtid, ax, ay);
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
 #pragma unroll
@@ -776,16 +732,17 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
 }
 
 // Waves of role B: gradient of slot 2, kept in registers across the tasks that share l2.
-__device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& u, BwdPrefetch& pf, BwdUTask t,
+__device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& u, BwdUTask t,
                                                 float2* __restrict__ part2_b) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2];
 #pragma unroll
     for (int i = 0; i < kBwdMaxTI; ++i) ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+    int par = 0, f2par = 0;
     for (int ti = u.task_begin; ti < u.task_end; ++ti) {
         BwdUTask cur;
-        float* cgp;
-        float2* g;
-        bwd_stage(c, u, ti, pf, t, cur, cgp, g);
+        const float* cgp;
+        const float2 *g, *f2;
+        bwd_stage(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
 #define CGNET_CALL_B(TI_, RW_) bwd_accum<2, TI_, RW_>(q, cgp, g, c.f1, c.rtid, ax, ay)
         CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_CALL_B)
@@ -799,11 +756,18 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
     }
 }
 
+// LDS map (bytes): [16 zero] f1 (f1cap) | f2 x2 (f2cap each) | table x2 (cgcap each) | [16 zero]
+// tile 0 (tcap) [16 zero] tile 1 (tcap) [16 zero].  Everything is cleared once, so positions a
+// tile read may touch just outside the tile hold finite values.
+__host__ __device__ inline size_t bwd_unit_lds(int f1cap, int f2cap, int cgcap, int tcap) {
+    return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + 16 + 2 * ((size_t)tcap + 16);
+}
+
 __global__ void __launch_bounds__(kThreads, 3)
-cg_backward_unit_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
-                        const float* __restrict__ CG, float2* __restrict__ part1, float2* __restrict__ part2,
+cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
+                        const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                         const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
-                        int nF, int nFF, int P2) {
+                        int nF, int nFp, int nFF, int P2, int f1cap, int f2cap, int cgcap, int tcap) {
     extern __shared__ __align__(16) unsigned char smem[];
     const BwdUnit u = units[blockIdx.x];
     const int b = blockIdx.y;
@@ -811,35 +775,67 @@ cg_backward_unit_kernel(const float2* __restrict__ F, const float2* __restrict__
     const int M1 = 2 * u.l1 + 1;
     const bool roleA = wave < u.nA;                  // wave-uniform
     BwdCtx c;
-    c.Fb = F + (size_t)b * nF;
+    c.Fp = Fp + (size_t)b * nFp;
     c.Gb = gFF + (size_t)b * nFF;
-    c.CG = CG;
+    c.CGP = CGP;
     c.tasks = tasks;
-    c.f1 = reinterpret_cast<float2*>(smem);
-    c.f2 = c.f1 + u.rows * (M1 + 1);
+    c.f1 = reinterpret_cast<float2*>(smem + 16);
+    c.f2 = reinterpret_cast<char*>(smem) + 16 + f1cap;
+    c.cg = c.f2 + 2 * f2cap;
+    c.tile = c.cg + 2 * cgcap + 16;
+    c.f2cap = f2cap; c.cgcap = cgcap; c.tcap = tcap;
     c.tid = tid;
     c.rtid = roleA ? tid : tid - 64 * u.nA;
 
-    BwdPrefetch pf;
-    const BwdUTask t0 = tasks[u.task_begin];
-    bwd_prefetch(pf, t0, u.rows, c.Gb, c.Fb, CG, tid);
     {
-        const float inv1 = 1.0f / (float)(M1 + 1);
-        for (int e = tid; e < u.rows * (M1 + 1); e += kThreads) {
-            const int row = (int)(((float)e + 0.5f) * inv1);
-            const int x = e - row * (M1 + 1);
-            c.f1[e] = x < M1 ? c.Fb[u.offF1 + row * M1 + x] : make_float2(0.f, 0.f);
-        }
+        const int n16 = (int)(bwd_unit_lds(f1cap, f2cap, cgcap, tcap) >> 4);
+        float4* z = reinterpret_cast<float4*>(smem);
+        for (int e = tid; e < n16; e += kThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
+    __syncthreads();                                 // the clearing stores precede every copy
+    const BwdUTask t0 = tasks[u.task_begin];
+    dma16(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
+    bwd_issue(c, u, t0, 0, 0);
 
-    // The two roles run the same sequence of barriers (two per task) from different code paths.
+    // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
         float2* dst = part1 + (size_t)b * nF + u.offF1;
-#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<TI_, RW_>(c, u, pf, t0, dst)
+#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<TI_, RW_>(c, u, t0, dst)
         CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
-        bwd_unit_loop_b(c, u, pf, t0, part2 + (size_t)b * P2);
+        bwd_unit_loop_b(c, u, t0, part2 + (size_t)b * P2);
+    }
+}
+
+// Builds the operands the unit kernel copies straight into LDS: fragments with one zero behind
+// every row (blocks below nbF) and every triple's table between kTabLo / kTabHi zero rows
+// (one block per triple).
+__global__ void __launch_bounds__(256)
+cg_backward_pad_kernel(const float2* __restrict__ F, const float* __restrict__ CG, float2* __restrict__ Fp,
+                       float* __restrict__ CGP, const int* __restrict__ meta, int L, int nF, int nFp, int B,
+                       int nbF) {
+    const int* cumF = meta;                 // L+2
+    const int* cumFp = meta + (L + 2);      // L+2
+    const int* tri = cumFp + (L + 2);       // 5 per triple
+    if ((int)blockIdx.x < nbF) {
+        const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (idx >= (size_t)B * nFp) return;
+        const int b = (int)(idx / nFp), e = (int)(idx % nFp);
+        int lam = 0;
+        while (lam < L && cumFp[lam + 1] <= e) ++lam;
+        const int rel = e - cumFp[lam], Mq = 2 * lam + 2;
+        const int t = rel / Mq, x = rel - t * Mq;
+        float2 v = make_float2(0.f, 0.f);
+        if (x < Mq - 1) v = F[(size_t)b * nF + cumF[lam] + t * (Mq - 1) + x];
+        Fp[idx] = v;
+    } else {
+        const int* m = tri + 5 * ((int)blockIdx.x - nbF);
+        const int cg_off = m[0], cgp_off = m[1], len = m[2], M = m[3], M2 = m[4];
+        for (int e = threadIdx.x; e < len; e += blockDim.x) {
+            const int x = e - kTabLo * M2;
+            CGP[cgp_off + e] = (x >= 0 && x < M * M2) ? CG[cg_off + x] : 0.f;
+        }
     }
 }
 
@@ -909,6 +905,7 @@ static void free_plan(cgnet_cg_plan* plan) {
     if (plan->d_bwd_units) (void)hipFree(plan->d_bwd_units);
     if (plan->d_bwd_utasks) (void)hipFree(plan->d_bwd_utasks);
     if (plan->d_bwd_combine) (void)hipFree(plan->d_bwd_combine);
+    if (plan->d_bwd_padmeta) (void)hipFree(plan->d_bwd_padmeta);
     delete plan;
 }
 
@@ -1093,11 +1090,20 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     }
 
     // ---- register-resident backward: units = (l1, range of t1 rows), tasks ordered by (l2, l)
-    std::vector<int> combine_meta;
+    std::vector<int> combine_meta, pad_meta;
     {
         bool ok = true;
         int P2 = 0;
         size_t lds_max = 0;
+        // fragments with one zero behind every row; every triple's table between zero rows
+        std::vector<int> cumFp(n1 + 1, 0), cgp_off(nllls + 1, 0);
+        for (int l = 0; l < n1; ++l) cumFp[l + 1] = cumFp[l] + h_t_F[l] * (2 * l + 2);
+        for (int i = 0; i < nllls; ++i) {
+            const long long len = ((long long)(2 * tl[i] + 1 + kTabLo + kTabHi) * (2 * tl2[i] + 1) + 1 + 3) & ~3LL;
+            if ((long long)cgp_off[i] + len > INT32_MAX) { ok = false; break; }
+            cgp_off[i + 1] = cgp_off[i] + (int)len;
+        }
+        int f1cap = 0, f2cap = 0, cgcap = 0, tcap = 0;
         std::vector<int> own1(n1, 0);
         std::vector<std::vector<int>> lam_offs(n1);
         std::vector<double> unit_cost;
@@ -1120,7 +1126,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 if (rows_c == prev_rows) continue;
                 prev_rows = rows_c;
                 long long max_tile = 0;
-                for (int i : tri) max_tile = std::max(max_tile, 8LL * rows_c * h_t_F[tl2[i]] * (2 * tl[i] + 1 + kPadLo + kPadHi));
+                for (int i : tri) max_tile = std::max(max_tile, 8LL * rows_c * h_t_F[tl2[i]] * (2 * tl[i] + 1));
                 if (max_tile > kBwdTileBytes && rows_c > 1) continue;
                 const int real_chunks = (tau1 + rows_c - 1) / rows_c;
                 for (int nA = 1; nA <= 3; ++nA) {
@@ -1172,17 +1178,21 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 u.l1 = l1;
                 u.rows = std::min(best.rows, tau1 - r0);
                 u.offF1 = p->cumF[l1] + r0 * M1;
+                u.offF1p = cumFp[l1] + r0 * (M1 + 1);
                 u.task_begin = (int)p->bwd_utasks.size();
                 u.nA = best.nA; u.TI = best.TI; u.RW = best.RW;
-                size_t task_lds = 0;
+                f1cap = std::max(f1cap, (int)align_up((size_t)8 * u.rows * (M1 + 1), 16));
                 for (int k = 0; k < nt; ++k) {
                     const int i = tri[k];
                     BwdUTask t;
                     t.l = tl[i]; t.l2 = tl2[i]; t.tau2 = h_t_F[tl2[i]];
-                    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1, Mp = M + kPadLo + kPadHi;
+                    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
                     t.offFF = p->cumFF[t.l] + (p->t_off[i] + r0 * t.tau2) * M;
                     t.offF2 = p->cumF[t.l2];
+                    t.offF2p = cumFp[t.l2];
                     t.cg_off = cgo[i];
+                    t.cgp_off = cgp_off[i];
+                    t.cgp_len = cgp_off[i + 1] - cgp_off[i];
                     t.first_of_l2 = (k == 0 || tl2[tri[k - 1]] != t.l2) ? 1 : 0;
                     t.last_of_l2 = (k + 1 == nt || tl2[tri[k + 1]] != t.l2) ? 1 : 0;
                     if (t.first_of_l2) {
@@ -1194,11 +1204,14 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     }
                     t.TI = best.bTI[k]; t.RW = best.bRW[k];
                     p->bwd_utasks.push_back(t);
-                    task_lds = std::max(task_lds, (size_t)8 * t.tau2 * (M2 + 1) + 4 * (size_t)((Mp * M2 + 2) & ~1) +
-                                                      (size_t)8 * u.rows * t.tau2 * Mp);
+                    const size_t tile_bytes = align_up((size_t)8 * u.rows * t.tau2 * M, 16);
+                    if (tile_bytes > kMaxLds) { ok = false; break; }
+                    f2cap = std::max(f2cap, (int)align_up((size_t)8 * t.tau2 * (M2 + 1), 16));
+                    cgcap = std::max(cgcap, 4 * t.cgp_len);
+                    tcap = std::max(tcap, (int)tile_bytes);
                 }
                 u.task_end = (int)p->bwd_utasks.size();
-                lds_max = std::max(lds_max, (size_t)8 * u.rows * (M1 + 1) + task_lds);
+                lds_max = bwd_unit_lds(f1cap, f2cap, cgcap, tcap);
                 p->bwd_units.push_back(u);
                 unit_cost.push_back(best.total);
             }
@@ -1206,7 +1219,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         // CGNET_BWD_GENERAL=1 forces the LDS-accumulator kernel (kept for shapes the unit scheme cannot hold)
         const char* force_general = getenv("CGNET_BWD_GENERAL");
         if (force_general && force_general[0] == '1') ok = false;
-        if (ok && !p->bwd_units.empty() && lds_max <= kMaxLds) {
+        if (ok && !p->bwd_units.empty() && lds_max <= kMaxUnitLds) {
             // longest units first
             std::vector<int> order(p->bwd_units.size());
             for (size_t k = 0; k < order.size(); ++k) order[k] = (int)k;
@@ -1216,6 +1229,15 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             p->bwd_units.swap(sorted);
             p->bwd_fast = true;
             p->bwd_P2 = P2;
+            p->bwd_nFp = cumFp[n1];
+            p->bwd_cgp_len = cgp_off[nllls];
+            p->bwd_f1cap = f1cap; p->bwd_f2cap = f2cap; p->bwd_cgcap = cgcap; p->bwd_tcap = tcap;
+            pad_meta.insert(pad_meta.end(), p->cumF.begin(), p->cumF.end());           // L+2
+            pad_meta.insert(pad_meta.end(), cumFp.begin(), cumFp.end());               // L+2
+            for (int i = 0; i < nllls; ++i) {
+                const int v[5] = {cgo[i], cgp_off[i], cgp_off[i + 1] - cgp_off[i], 2 * tl[i] + 1, 2 * tl2[i] + 1};
+                pad_meta.insert(pad_meta.end(), v, v + 5);
+            }
             if (const char* dbg = getenv("CGNET_DEBUG"); dbg && dbg[0] == '1') {
                 fprintf(stderr, "[cgnet] backward units=%zu tasks=%zu P2=%d lds=%zu\n", p->bwd_units.size(),
                         p->bwd_utasks.size(), P2, lds_max);
@@ -1255,6 +1277,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         CGNET_HIP(hipMemcpy(p->d_bwd_utasks, p->bwd_utasks.data(), sizeof(BwdUTask) * p->bwd_utasks.size(), hipMemcpyHostToDevice));
         CGNET_HIP(hipMalloc((void**)&p->d_bwd_combine, sizeof(int) * combine_meta.size()));
         CGNET_HIP(hipMemcpy(p->d_bwd_combine, combine_meta.data(), sizeof(int) * combine_meta.size(), hipMemcpyHostToDevice));
+        CGNET_HIP(hipMalloc((void**)&p->d_bwd_padmeta, sizeof(int) * pad_meta.size()));
+        CGNET_HIP(hipMemcpy(p->d_bwd_padmeta, pad_meta.data(), sizeof(int) * pad_meta.size(), hipMemcpyHostToDevice));
         if (p->bwd_fast_lds > 64 * 1024)
             CGNET_HIP(hipFuncSetAttribute((const void*)cg_backward_unit_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_fast_lds));
     }
@@ -1353,7 +1377,9 @@ extern "C" size_t cgnet_sparse_backward_workspace(const cgnet_cg_plan* plan, int
     if (!plan || B <= 0) return 0;
     if (plan->bwd_fast)
         return align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256) +
-               align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256);
+               align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256) +
+               align_up(sizeof(float) * 2 * (size_t)plan->bwd_nFp * B, 256) +
+               align_up(sizeof(float) * (size_t)plan->bwd_cgp_len, 256);
     const int ng = bwd_groups_for(plan, B);
     if (ng <= 1) return 0;
     return align_up(sizeof(float) * 2 * (size_t)plan->nF * B * ng, 256);
@@ -1381,10 +1407,19 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
                   "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if (plan->bwd_fast) {
         float2* part1 = (float2*)d_workspace;
-        float2* part2 = (float2*)((char*)d_workspace + align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256));
+        float2* part2 = (float2*)((char*)part1 + align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256));
+        float2* Fp = (float2*)((char*)part2 + align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256));
+        float* CGP = (float*)((char*)Fp + align_up(sizeof(float) * 2 * (size_t)plan->bwd_nFp * B, 256));
+        CGNET_REQUIRE(((uintptr_t)d_workspace & 15) == 0, CGNET_ERR_ARG, "workspace must be 16-byte aligned");
+        const size_t npad = (size_t)plan->bwd_nFp * B;
+        const int nbF = (int)((npad + 255) / 256);
+        CGNET_LAUNCH(cg_backward_pad_kernel, dim3((unsigned)(nbF + plan->nllls)), dim3(256), 0, s,
+                     (const float2*)d_F, d_CG, Fp, CGP, plan->d_bwd_padmeta, plan->L, plan->nF, plan->bwd_nFp, B, nbF);
+        CGNET_HIP(hipGetLastError());
         CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)plan->bwd_units.size(), B), dim3(kThreads),
-                     plan->bwd_fast_lds, s, (const float2*)d_F, (const float2*)d_gFF, d_CG, part1, part2,
-                     plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->nFF, plan->bwd_P2);
+                     plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
+                     plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
+                     plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap);
         CGNET_HIP(hipGetLastError());
         const size_t n = (size_t)plan->nF * B;
         CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
