@@ -97,7 +97,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kFwdTileBytes = 32 * 1024;
-constexpr int kBwdTileBytes = 16 * 1024;
+constexpr int kBwdTileBytes = 14 * 1024;
 constexpr int kMaxTileChannels = 4 * kThreads;   // statistics: at most four channels per thread
 constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
@@ -763,7 +763,7 @@ __host__ __device__ inline size_t bwd_unit_lds(int f1cap, int f2cap, int cgcap, 
     return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + 16 + 2 * ((size_t)tcap + 16);
 }
 
-__global__ void __launch_bounds__(kThreads, 3)
+__global__ void __launch_bounds__(kThreads, 4)
 cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
                         const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                         const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
