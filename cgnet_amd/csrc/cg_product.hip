@@ -484,6 +484,25 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 }
 
 // ---- register-resident backward ------------------------------------------------------------
+// LDS byte address of a pointer into shared memory, and typed reads through such addresses.
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(3))) v2f_t* lds_f2_ptr;
+typedef const __attribute__((address_space(3))) float* lds_f_ptr;
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// complex entry k behind LDS byte address a
+__device__ __forceinline__ float2 lds_c(unsigned a, int k) {
+    const v2f_t v = ((lds_f2_ptr)(uintptr_t)a)[k];
+    return make_float2(v.x, v.y);
+}
+__device__ __forceinline__ lds_f_ptr lds_f(unsigned a) { return (lds_f_ptr)(uintptr_t)a; }
+// Keeps a per-lane value in one register: the optimiser may not split it into base + offset again.
+__device__ __forceinline__ unsigned opaque(unsigned v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 struct BwdGeom { int l, l1, l2, rows, tau2; };
 constexpr int kBwdMaxTI = 4;   // output channels per thread
 // Zero rows before / after the staged CG table.  The two m outputs of a thread and the two-step
@@ -520,54 +539,75 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
 #pragma unroll
     for (int i = 0; i < TI; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
     const int col0 = min(mo0, M2 - 1), col1 = min(mo0 + 1, M2 - 1);
+    // Per-lane LDS byte addresses, advanced by constants inside the loop.  Coefficients of the
+    // step pair (ir, ir+1):  c0 = T[p][k0], c1 = T[p+1][k1], c0' = T[p+1][k0'], c1' = T[p+2][k1']
+    // with p the table row of (mo0, ir); slot 1: k = ir (k0' = k1' = ir+1), slot 2: k0 = col0, k1 = col1.
+    const unsigned c_step = (SLOT == 1) ? 8u * (M2 + 1) : 8u * M2;     // two rows (and two columns) per pair
     for (int r = lane_r; r < n_r; r += RW) {
-        const float2* frow = fr + r * (M_r + 1);      // rows carry one trailing zero
-        const float2* gb = g + r * g_sr + (mo0 - d);
-        const float* cb = cgp + (kTabLo + mo0 - d) * M2;
+        unsigned gp[TI];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) gp[i] = lds_addr(g + r * g_sr + (mo0 - d) + go[i] + ir_lo);
+        unsigned fp = lds_addr(fr + r * (M_r + 1) + ir_lo);           // rows carry one trailing zero
+        const float* cb = cgp + (kTabLo + mo0 - d + ir_lo) * M2;       // table row of (mo0, ir_lo)
+        unsigned ca = lds_addr(cb + ((SLOT == 1) ? ir_lo : col0));     // c0
+        unsigned cbn = lds_addr(cb + M2 + ((SLOT == 1) ? ir_lo : col1));   // c1 (slot 1: c0' is the next float)
+        unsigned cc = lds_addr(cb + 2 * M2 + ((SLOT == 1) ? ir_lo + 1 : col1));  // c1'
+        unsigned cd = lds_addr(cb + M2 + col0);                        // slot 2: c0'
+        const unsigned f_end = fp + 8u * (unsigned)(ir_hi - ir_lo);
+        const bool any = ir_hi >= ir_lo;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) gp[i] = opaque(gp[i]);
+        fp = opaque(fp); ca = opaque(ca); cbn = opaque(cbn); cc = opaque(cc);
+        if (SLOT == 2) cd = opaque(cd);
         float2 e0[TI], e1[TI];
 #pragma unroll
-        for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir_lo];
-        for (int ir = ir_lo; ir <= ir_hi; ir += 2) {
+        for (int i = 0; i < TI; ++i) e0[i] = lds_c(gp[i], 0);
+        if (any) {
+#pragma unroll 2
+            for (; fp <= f_end; ) {
+                float2 e2[TI];
 #pragma unroll
-            for (int i = 0; i < TI; ++i) e1[i] = gb[go[i] + ir + 1];
-            {
-                const float2 f = frow[ir];
-                const float c0 = (SLOT == 1) ? cb[ir * M2 + ir] : cb[ir * M2 + col0];
-                const float c1 = (SLOT == 1) ? cb[(ir + 1) * M2 + ir] : cb[(ir + 1) * M2 + col1];
-                const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
+                for (int i = 0; i < TI; ++i) { e1[i] = lds_c(gp[i], 1); e2[i] = lds_c(gp[i], 2); }
+                const float2 fa = lds_c(fp, 0), fb = lds_c(fp, 1);
+                const float c0 = lds_f(ca)[0];
+                const float c1 = lds_f(cbn)[0];
+                const float d0 = (SLOT == 1) ? lds_f(cbn)[1] : lds_f(cd)[0];
+                const float d1 = lds_f(cc)[0];
+                {
+                    const float c0x = c0 * fa.x, c0y = -c0 * fa.y, c1x = c1 * fa.x, c1y = -c1 * fa.y;
 #pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    ax[i][0] = fmaf(e0[i].x, c0x, ax[i][0]);
-                    ax[i][0] = fmaf(-e0[i].y, c0y, ax[i][0]);
-                    ay[i][0] = fmaf(e0[i].x, c0y, ay[i][0]);
-                    ay[i][0] = fmaf(e0[i].y, c0x, ay[i][0]);
-                    ax[i][1] = fmaf(e1[i].x, c1x, ax[i][1]);
-                    ax[i][1] = fmaf(-e1[i].y, c1y, ax[i][1]);
-                    ay[i][1] = fmaf(e1[i].x, c1y, ay[i][1]);
-                    ay[i][1] = fmaf(e1[i].y, c1x, ay[i][1]);
+                    for (int i = 0; i < TI; ++i) {
+                        ax[i][0] = fmaf(e0[i].x, c0x, ax[i][0]);
+                        ax[i][0] = fmaf(-e0[i].y, c0y, ax[i][0]);
+                        ay[i][0] = fmaf(e0[i].x, c0y, ay[i][0]);
+                        ay[i][0] = fmaf(e0[i].y, c0x, ay[i][0]);
+                        ax[i][1] = fmaf(e1[i].x, c1x, ax[i][1]);
+                        ax[i][1] = fmaf(-e1[i].y, c1y, ax[i][1]);
+                        ay[i][1] = fmaf(e1[i].x, c1y, ay[i][1]);
+                        ay[i][1] = fmaf(e1[i].y, c1x, ay[i][1]);
+                    }
                 }
-            }
+                {
+                    // past the valid range either the fragment (padded row) or the table row
+                    // (padded) is zero, so no masking is needed
+                    const float c0x = d0 * fb.x, c0y = -d0 * fb.y, c1x = d1 * fb.x, c1y = -d1 * fb.y;
 #pragma unroll
-            for (int i = 0; i < TI; ++i) e0[i] = gb[go[i] + ir + 2];
-            {
-                // past the valid range either the fragment (padded row) or the table row (padded)
-                // is zero, so no masking is needed
-                const int ir1 = ir + 1;
-                const float2 f = frow[ir1];
-                const float c0 = (SLOT == 1) ? cb[ir1 * M2 + ir1] : cb[ir1 * M2 + col0];
-                const float c1 = (SLOT == 1) ? cb[(ir1 + 1) * M2 + ir1] : cb[(ir1 + 1) * M2 + col1];
-                const float c0x = c0 * f.x, c0y = -c0 * f.y, c1x = c1 * f.x, c1y = -c1 * f.y;
-#pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    ax[i][0] = fmaf(e1[i].x, c0x, ax[i][0]);
-                    ax[i][0] = fmaf(-e1[i].y, c0y, ax[i][0]);
-                    ay[i][0] = fmaf(e1[i].x, c0y, ay[i][0]);
-                    ay[i][0] = fmaf(e1[i].y, c0x, ay[i][0]);
-                    ax[i][1] = fmaf(e0[i].x, c1x, ax[i][1]);
-                    ax[i][1] = fmaf(-e0[i].y, c1y, ax[i][1]);
-                    ay[i][1] = fmaf(e0[i].x, c1y, ay[i][1]);
-                    ay[i][1] = fmaf(e0[i].y, c1x, ay[i][1]);
+                    for (int i = 0; i < TI; ++i) {
+                        ax[i][0] = fmaf(e1[i].x, c0x, ax[i][0]);
+                        ax[i][0] = fmaf(-e1[i].y, c0y, ax[i][0]);
+                        ay[i][0] = fmaf(e1[i].x, c0y, ay[i][0]);
+                        ay[i][0] = fmaf(e1[i].y, c0x, ay[i][0]);
+                        ax[i][1] = fmaf(e2[i].x, c1x, ax[i][1]);
+                        ax[i][1] = fmaf(-e2[i].y, c1y, ax[i][1]);
+                        ay[i][1] = fmaf(e2[i].x, c1y, ay[i][1]);
+                        ay[i][1] = fmaf(e2[i].y, c1x, ay[i][1]);
+                    }
                 }
+#pragma unroll
+                for (int i = 0; i < TI; ++i) { e0[i] = e2[i]; gp[i] += 16u; }
+                fp += 16u;
+                ca += c_step; cbn += c_step; cc += c_step;
+                if (SLOT == 2) cd += c_step;
             }
         }
     }
