@@ -108,7 +108,38 @@ __host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
     return 8 * ((size_t)t.rows * t.tau2 * M + (size_t)t.rows * M1 + (size_t)t.tau2 * M2) + 4 * M * M2;
 }
 
+// ---------------------------------------------------------------------------- LDS addressing
+// LDS byte address of a pointer into shared memory, and typed reads through such addresses.
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(3))) v2f_t* lds_f2_ptr;
+typedef const __attribute__((address_space(3))) float* lds_f_ptr;
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// complex entry k behind LDS byte address a
+__device__ __forceinline__ float2 lds_c(unsigned a, int k) {
+    const v2f_t v = ((lds_f2_ptr)(uintptr_t)a)[k];
+    return make_float2(v.x, v.y);
+}
+__device__ __forceinline__ lds_f_ptr lds_f(unsigned a) { return (lds_f_ptr)(uintptr_t)a; }
+// Keeps a per-lane value in one register: the optimiser may not split it into base + offset again.
+__device__ __forceinline__ unsigned opaque(unsigned v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+
 // ------------------------------------------------------------------------------------ forward
+// Square root from the hardware reciprocal square root plus one Newton step (error below one
+// ulp); sqrt_refined(0) = 0.
+__device__ __forceinline__ float sqrt_refined(float n) {
+    const float y = __builtin_amdgcn_rsqf(fmaxf(n, 1e-37f));
+    const float s = n * y;
+    return fmaf(fmaf(-s, s, n), 0.5f * y, s);
+}
+
+// One item = one m of a TI x TJ tile of channels.  Items are ordered m-major, so the lanes of a
+// wave work on neighbouring m (similar numbers of terms) of all channel tiles.
 template <int TI, int TJ>
 __device__ __forceinline__ void fwd_tiles(const CgTask& t, const float* __restrict__ cg,
                                           const float2* __restrict__ f1, const float2* __restrict__ f2,
@@ -116,40 +147,46 @@ __device__ __forceinline__ void fwd_tiles(const CgTask& t, const float* __restri
     const int l = t.l, l1 = t.l1, l2 = t.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int nT1 = t.nT1, nT2 = t.nT2, rows = t.rows, tau2 = t.tau2;
-    const int nitems = nT1 * nT2 * M;
+    const int ntiles = nT1 * nT2;
+    const int nitems = ntiles * M;
     for (int item = threadIdx.x; item < nitems; item += kThreads) {
-        const int mm = item % M;
-        const int tt = item / M;
+        const int mm = item / ntiles;
+        const int tt = item - mm * ntiles;
         const int tj = tt % nT2, ti = tt / nT2;
         const int m = mm - l;
         const int lo = max(-l2, m - l1), hi = min(l2, m + l1);
         float ar[TI][TJ], ai[TI][TJ];
-        int r1[TI], r2[TJ];
+        unsigned pa[TI], pb[TJ];
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
-            r1[i] = min(ti + nT1 * i, rows - 1) * M1 + (m + l1);
+            pa[i] = opaque(lds_addr(f1 + min(ti + nT1 * i, rows - 1) * M1 + (m + l1) - lo));   // walks down
 #pragma unroll
             for (int j = 0; j < TJ; ++j) ar[i][j] = ai[i][j] = 0.f;
         }
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) r2[j] = min(tj + nT2 * j, tau2 - 1) * M2 + l2;
-        const float* cgrow = cg + mm * M2 + l2;
-        for (int m2 = lo; m2 <= hi; ++m2) {
-            const float c = cgrow[m2];
-            float2 b[TJ];
+        for (int j = 0; j < TJ; ++j) pb[j] = opaque(lds_addr(f2 + min(tj + nT2 * j, tau2 - 1) * M2 + l2 + lo));
+        unsigned pc = opaque(lds_addr(cg + mm * M2 + l2 + lo));
+        const unsigned pc_end = pc + 4u * (unsigned)(hi - lo);
+        if (hi >= lo) {
+#pragma unroll 2
+            for (; pc <= pc_end; pc += 4u) {
+                const float c = lds_f(pc)[0];
+                float2 b[TJ];
 #pragma unroll
-            for (int j = 0; j < TJ; ++j) b[j] = f2[r2[j] + m2];
+                for (int j = 0; j < TJ; ++j) { b[j] = lds_c(pb[j], 0); pb[j] += 8u; }
 #pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                float2 a = f1[r1[i] - m2];
-                a.x *= c;
-                a.y *= c;
+                for (int i = 0; i < TI; ++i) {
+                    float2 a = lds_c(pa[i], 0);
+                    pa[i] -= 8u;
+                    a.x *= c;
+                    a.y *= c;
 #pragma unroll
-                for (int j = 0; j < TJ; ++j) {
-                    ar[i][j] = fmaf(a.x, b[j].x, ar[i][j]);
-                    ar[i][j] = fmaf(-a.y, b[j].y, ar[i][j]);
-                    ai[i][j] = fmaf(a.x, b[j].y, ai[i][j]);
-                    ai[i][j] = fmaf(a.y, b[j].x, ai[i][j]);
+                    for (int j = 0; j < TJ; ++j) {
+                        ar[i][j] = fmaf(a.x, b[j].x, ar[i][j]);
+                        ar[i][j] = fmaf(-a.y, b[j].y, ar[i][j]);
+                        ai[i][j] = fmaf(a.x, b[j].y, ai[i][j]);
+                        ai[i][j] = fmaf(a.y, b[j].x, ai[i][j]);
+                    }
                 }
             }
         }
@@ -220,7 +257,7 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
                         const float2 z = out[ch * M + mm];
                         const float n = fmaf(z.x, z.x, z.y * z.y);
                         q += n;
-                        a += sqrtf(n);
+                        a += sqrt_refined(n);
                     }
                     s1[k] += (double)a;
                     s2[k] += (double)q;
@@ -484,25 +521,6 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 }
 
 // ---- register-resident backward ------------------------------------------------------------
-// LDS byte address of a pointer into shared memory, and typed reads through such addresses.
-typedef float v2f_t __attribute__((ext_vector_type(2)));
-typedef const __attribute__((address_space(3))) v2f_t* lds_f2_ptr;
-typedef const __attribute__((address_space(3))) float* lds_f_ptr;
-__device__ __forceinline__ unsigned lds_addr(const void* p) {
-    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-// complex entry k behind LDS byte address a
-__device__ __forceinline__ float2 lds_c(unsigned a, int k) {
-    const v2f_t v = ((lds_f2_ptr)(uintptr_t)a)[k];
-    return make_float2(v.x, v.y);
-}
-__device__ __forceinline__ lds_f_ptr lds_f(unsigned a) { return (lds_f_ptr)(uintptr_t)a; }
-// Keeps a per-lane value in one register: the optimiser may not split it into base + offset again.
-__device__ __forceinline__ unsigned opaque(unsigned v) {
-    asm volatile("" : "+v"(v));
-    return v;
-}
-
 struct BwdGeom { int l, l1, l2, rows, tau2; };
 constexpr int kBwdMaxTI = 4;   // output channels per thread
 // Zero rows before / after the staged CG table.  The two m outputs of a thread and the two-step
