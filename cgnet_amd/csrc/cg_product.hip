@@ -103,10 +103,6 @@ constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
 constexpr size_t kMaxUnitLds = 64 * 1024;       // unit backward: LDS-direct copies address the first 64 KB
 
-__host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
-    const size_t M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
-    return 8 * ((size_t)t.rows * t.tau2 * M + (size_t)t.rows * M1 + (size_t)t.tau2 * M2) + 4 * M * M2;
-}
 
 // ---------------------------------------------------------------------------- LDS addressing
 // LDS byte address of a pointer into shared memory, and typed reads through such addresses.
@@ -127,6 +123,30 @@ __device__ __forceinline__ unsigned opaque(unsigned v) {
     asm volatile("" : "+v"(v));
     return v;
 }
+
+
+// ---- operand staging: global memory -> LDS without passing through registers ----------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// Starts the copy of `nchunks` 16-byte pieces from `src` (8-byte aligned is enough) to the LDS
+// address `dst` (16-byte aligned).  Lane i of a wave lands 16*i bytes behind the wave's first
+// piece, so consecutive threads fill consecutive pieces.  Nothing may read the destination
+// before dma_wait() and a barrier.
+__device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
+    const char* s = reinterpret_cast<const char*>(src);
+    char* d = reinterpret_cast<char*>(dst);
+    for (int e = tid; e < nchunks; e += kThreads)
+        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
+}
+
+// One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1.
+__device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, int tid) {
+    if (tid < 2)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
+}
+
+// All copies this wave has started have landed (vmcnt == 0).
+__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
 
 // ------------------------------------------------------------------------------------ forward
@@ -213,6 +233,17 @@ __device__ __forceinline__ void fwd_dispatch_j(const CgTask& t, const float* cg,
     }
 }
 
+// LDS of the forward kernel: two fragment buffers (slab of l1 rows, slab of l2) | output tile | table
+__host__ __device__ inline size_t fwd_frag_lds(const CgTask& t) {
+    const size_t M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
+    return ((8 * (size_t)t.rows * M1 + 15) & ~(size_t)15) + ((8 * (size_t)t.tau2 * M2 + 15) & ~(size_t)15);
+}
+
+__host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
+    const size_t M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
+    return ((8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15) + 2 * fwd_frag_lds(t) + 4 * M * M2;
+}
+
 __global__ void __launch_bounds__(kThreads)
 cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const float* __restrict__ CG,
                   const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
@@ -222,22 +253,37 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
     const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
     const int nch = t.rows * t.tau2;
     const int nout = nch * M, n1 = t.rows * M1, n2 = t.tau2 * M2, ncg = M * M2;
-    float2* out = reinterpret_cast<float2*>(smem);
-    float2* f1 = out + nout;
-    float2* f2 = f1 + n1;
-    float* cg = reinterpret_cast<float*>(f2 + n2);
+    const size_t out_bytes = (8 * (size_t)nout + 15) & ~(size_t)15;
+    const size_t f1_bytes = (8 * (size_t)n1 + 15) & ~(size_t)15;
+    const size_t frag_bytes = fwd_frag_lds(t);
+    unsigned char* frag = smem;                                   // [2][frag_bytes], the LDS-direct copy targets
+    float2* out = reinterpret_cast<float2*>(smem + 2 * frag_bytes);
+    float* cg = reinterpret_cast<float*>(smem + 2 * frag_bytes + out_bytes);
     const int tid = threadIdx.x;
 
-    for (int e = tid; e < ncg; e += kThreads) cg[e] = CG[t.cg_off + e];
+    // fragments of sample b -> buffer `par`, straight into LDS
+    auto issue = [&](int b, int par) {
+        const float2* Fb = F + (size_t)b * nF;
+        unsigned char* d1 = frag + par * frag_bytes;
+        unsigned char* d2 = d1 + f1_bytes;
+        dma16(Fb + t.offF1, d1, n1 >> 1, tid);
+        if (n1 & 1) dma8(Fb + t.offF1 + (n1 - 1), d1 + 8 * (size_t)(n1 - 1), tid);
+        dma16(Fb + t.offF2, d2, n2 >> 1, tid);
+        if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
+    };
 
     double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};
     const int b0 = blockIdx.y * samples_per_group;
     const int b1 = min(B, b0 + samples_per_group);
-    for (int b = b0; b < b1; ++b) {
-        const float2* Fb = F + (size_t)b * nF;
-        for (int e = tid; e < n1; e += kThreads) f1[e] = Fb[t.offF1 + e];
-        for (int e = tid; e < n2; e += kThreads) f2[e] = Fb[t.offF2 + e];
-        __syncthreads();
+    if (b0 < b1) issue(b0, 0);
+    for (int e = tid; e < ncg; e += kThreads) cg[e] = CG[t.cg_off + e];
+    int par = 0;
+    for (int b = b0; b < b1; ++b, par ^= 1) {
+        dma_wait();
+        __syncthreads();       // this sample's fragments landed; the previous tile has been copied out
+        if (b + 1 < b1) issue(b + 1, par ^ 1);
+        const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
+        const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
         switch (t.TI) {
             case 1: fwd_dispatch_j<1>(t, cg, f1, f2, out); break;
             case 2: fwd_dispatch_j<2>(t, cg, f1, f2, out); break;
@@ -245,8 +291,17 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
             default: fwd_dispatch_j<4>(t, cg, f1, f2, out); break;
         }
         __syncthreads();
+        // tile -> FF with 16-byte stores from the first 16-byte boundary on
         float2* dst = FF + (size_t)b * nFF + t.offFF;
-        for (int e = tid; e < nout; e += kThreads) dst[e] = out[e];
+        const int head = min(nout, (int)((reinterpret_cast<uintptr_t>(dst) >> 3) & 1));
+        const int npair = (nout - head) >> 1;
+        float4* dst4 = reinterpret_cast<float4*>(dst + head);
+        for (int e = tid; e < npair; e += kThreads) {
+            const float2 u = out[head + 2 * e], v = out[head + 2 * e + 1];
+            dst4[e] = make_float4(u.x, u.y, v.x, v.y);
+        }
+        if (tid == 0 && head) dst[0] = out[0];
+        if (tid == 1 && ((nout - head) & 1)) dst[nout - 1] = out[nout - 1];
         if (stats_part) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -264,7 +319,6 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
                 }
             }
         }
-        __syncthreads();
     }
     if (stats_part) {
 #pragma unroll
@@ -688,29 +742,6 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         default: { CALL(4, 16); } break;                                         \
     }
 
-// ---- operand staging: global memory -> LDS without passing through registers ----------------
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-
-// Starts the copy of `nchunks` 16-byte pieces from `src` (8-byte aligned is enough) to the LDS
-// address `dst` (16-byte aligned).  Lane i of a wave lands 16*i bytes behind the wave's first
-// piece, so consecutive threads fill consecutive pieces.  Nothing may read the destination
-// before dma_wait() and a barrier.
-__device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
-    const char* s = reinterpret_cast<const char*>(src);
-    char* d = reinterpret_cast<char*>(dst);
-    for (int e = tid; e < nchunks; e += kThreads)
-        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
-}
-
-// One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1.
-__device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, int tid) {
-    if (tid < 2)
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
-}
-
-// All copies this wave has started have landed (vmcnt == 0).
-__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
-
 struct BwdCtx {
     const float2* Fp;          // this sample's fragments, rows padded with one zero
     const float2* Gb;          // this sample's gFF
@@ -1103,7 +1134,11 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                (long long)b.rows * b.tau2 * (2 * b.l + 1) * (2 * b.l2 + 1);
     });
     size_t fl = 0, bl = 0;
-    for (const CgTask& t : p->fwd_tasks) fl = std::max(fl, fwd_task_lds(t));
+    for (const CgTask& t : p->fwd_tasks) {
+        fl = std::max(fl, fwd_task_lds(t));
+        CGNET_REQUIRE(2 * fwd_frag_lds(t) <= kMaxUnitLds, CGNET_ERR_UNSUPPORTED,
+                      "fragment slabs of %zu bytes exceed the LDS staging window", 2 * fwd_frag_lds(t));
+    }
     for (const CgTask& t : p->bwd_tasks) bl = std::max(bl, bwd_task_lds(t));
     p->fwd_lds = align_up(fl, 16);
     p->bwd_lds = align_up(bl, 16) + 8 * (size_t)p->nF;
