@@ -93,5 +93,7 @@ def kernel_times():
     for i in range(n):
         ms, cnt = ctypes.c_double(), ctypes.c_int()
         check(lib.cgnet_profile_get(i, buf, len(buf), ctypes.byref(ms), ctypes.byref(cnt)))
-        out[buf.value.decode()] = (ms.value, cnt.value)
+        name = buf.value.decode().split("<")[0]      # template instances of one kernel are added up
+        prev = out.get(name, (0.0, 0))
+        out[name] = (prev[0] + ms.value, prev[1] + cnt.value)
     return out

@@ -125,28 +125,6 @@ __device__ __forceinline__ unsigned opaque(unsigned v) {
 }
 
 
-// ---- operand staging: global memory -> LDS without passing through registers ----------------
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-
-// Starts the copy of `nchunks` 16-byte pieces from `src` (8-byte aligned is enough) to the LDS
-// address `dst` (16-byte aligned).  Lane i of a wave lands 16*i bytes behind the wave's first
-// piece, so consecutive threads fill consecutive pieces.  Nothing may read the destination
-// before dma_wait() and a barrier.
-__device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
-    const char* s = reinterpret_cast<const char*>(src);
-    char* d = reinterpret_cast<char*>(dst);
-    for (int e = tid; e < nchunks; e += kThreads)
-        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
-}
-
-// One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1.
-__device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, int tid) {
-    if (tid < 2)
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
-}
-
-// All copies this wave has started have landed (vmcnt == 0).
-__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
 
 // ------------------------------------------------------------------------------------ forward
@@ -266,9 +244,9 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
         const float2* Fb = F + (size_t)b * nF;
         unsigned char* d1 = frag + par * frag_bytes;
         unsigned char* d2 = d1 + f1_bytes;
-        dma16(Fb + t.offF1, d1, n1 >> 1, tid);
+        dma16<kThreads>(Fb + t.offF1, d1, n1 >> 1, tid);
         if (n1 & 1) dma8(Fb + t.offF1 + (n1 - 1), d1 + 8 * (size_t)(n1 - 1), tid);
-        dma16(Fb + t.offF2, d2, n2 >> 1, tid);
+        dma16<kThreads>(Fb + t.offF2, d2, n2 >> 1, tid);
         if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
     };
 
@@ -761,10 +739,10 @@ __device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, con
     const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
     const int ntile = u.rows * t.tau2 * M;
     char* tile = c.tile + par * (c.tcap + 16);
-    dma16(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
+    dma16<kThreads>(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
     if (ntile & 1) dma8(c.Gb + t.offFF + (ntile - 1), tile + 8 * (size_t)(ntile - 1), c.tid);
-    dma16(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
-    if (t.first_of_l2) dma16(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
+    dma16<kThreads>(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
+    if (t.first_of_l2) dma16<kThreads>(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
 }
 
 // Per-task prologue of both roles.  On entry `t` is the task whose copies were started one
@@ -883,7 +861,7 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
     }
     __syncthreads();                                 // the clearing stores precede every copy
     const BwdUTask t0 = tasks[u.task_begin];
-    dma16(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
+    dma16<kThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
     bwd_issue(c, u, t0, 0, 0);
 
     // The two roles run the same sequence of barriers (one per task) from different code paths.

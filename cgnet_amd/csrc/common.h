@@ -53,4 +53,30 @@ private:
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                    \
     } while (0)
 
+// ---- global memory -> LDS copies that bypass the registers (gfx950 LDS-direct loads) ----------
+// The hardware places lane i of a wave 16*i (4*i for dword copies) bytes behind the LDS address
+// the wave passes; the copy is tracked by vmcnt.  Nothing may read the destination before the
+// issuing wave has executed dma_wait() and a barrier has been passed.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// Starts the copy of `nchunks` 16-byte pieces from `src` (8-byte aligned is enough) to the LDS
+// address `dst` (16-byte aligned) by NT cooperating threads, `tid` = 0 .. NT-1 (NT a multiple of 64).
+template <int NT>
+__device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
+    const char* s = reinterpret_cast<const char*>(src);
+    char* d = reinterpret_cast<char*>(dst);
+    for (int e = tid; e < nchunks; e += NT)
+        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
+}
+
+// One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1 of the
+// wave whose threads have tid 0 and 1.
+__device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, int tid) {
+    if (tid < 2)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
+}
+
+// All copies (and loads) this wave has started have landed (vmcnt == 0).
+__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+
 }  // namespace cgnet

@@ -50,11 +50,12 @@ struct cgnet_wmm_plan {
     int ap_blocks = 0;     // 64-float blocks of the packed operand of the FF-gradient kernel
     bool gff_mfma = true;  // every degree has t_O <= 16 (the operand then fits eight registers)
     int gw_ff_cap = 2, gw_go_cap = 2;   // LDS capacities (complex entries) of one stage of the weight-gradient kernel
-    int fwd_stage_cap = 2;              // LDS capacity (complex entries) of one stage of the forward kernel
+    int fwd_stage_cap = 16;             // LDS bytes of one stage of one wave of the forward kernel
     int gff_out_cap = 4, gff_go_cap = 2; // LDS capacities of the FF-gradient kernel (real entries / complex entries)
     int maxS = 1, maxG = 1;
     std::vector<cgnet::WmmDeg> degs;
-    std::vector<cgnet::WmmFwdUnit> fwd_units;
+    std::vector<cgnet::WmmFwdUnit> fwd_units;   // units of degrees with NC <= 3 first
+    int fwd_units_small = 0;
     std::vector<cgnet::WmmChanUnit> gw_units, gw_units_rc0, gff_units, stat_units;
     std::vector<int> cumO_all, cumFF_all;   // L+2 entries, for element -> degree lookups
     cgnet::WmmDeg* d_degs = nullptr;
@@ -147,17 +148,18 @@ __global__ void __launch_bounds__(256)
 pack_w_forward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                       const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int total_blocks) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int blk = idx >> 6, lane = idx & 63;
+    const int blk = idx >> 6;
     if (blk >= total_blocks) return;
     int di = 0;
     while (di + 1 < ndeg && degs[di + 1].wp_base <= blk) ++di;
     const WmmDeg d = degs[di];
-    const int rel = blk - d.wp_base;             // ((ks * nrc) + rc) * 2 + tile
-    const int tile = rel & 1;
-    const int rc = (rel >> 1) % d.nrc;
-    const int ks = (rel >> 1) / d.nrc;
+    // 256 floats per (block of 8 channels, row chunk): lane-major, 4 per lane = (step, re/im rows)
+    const int rel = idx - d.wp_base * 64;
+    const int sub = rel & 3, lane = (rel >> 2) & 63, grp = rel >> 8;
+    const int tile = sub & 1, step = sub >> 1;
+    const int rc = grp % d.nrc, kb = grp / d.nrc;
     const int row = lane & 15, kk = lane >> 4;
-    const int to = rc * 16 + row, c = ks * 4 + kk;
+    const int to = rc * 16 + row, c = kb * 8 + step * 4 + kk;
     float v = 0.f;
     if (to < d.tO && c < d.K) {
         const float2 w = W[d.cumW + (size_t)to * d.K + c];
@@ -235,137 +237,100 @@ struct Run16 {
     }
 };
 
-// Forward mixing.  A work-group owns G whole samples of one degree and a slice of the channels.
-// Per stage it streams kFwdKC channels of every sample (one contiguous run each) through LDS
-// with 16-byte lane-contiguous loads, double buffered; wave w owns complex columns
-// 32w .. 32w+31 of the G*M columns and reads its operands from LDS in matrix-core order.  The
-// weights come packed in lane order straight from L2, one stage ahead.
-constexpr int kFwdKC = 16;       // channels per stage (a multiple of 4)
-constexpr int kFwdRegs = 4;      // float4 registers per thread and stage: 4 x 256 x 2 = 2048 complex
-
-__global__ void __launch_bounds__(kThreads, 4)
-wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
-                   const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO,
-                   int stage_cap) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    float2* lds = reinterpret_cast<float2*>(smem);                // [2][stage_cap]
-    const WmmFwdUnit u = units[blockIdx.x];
-    const WmmDeg d = degs[u.deg];
-    const int b0 = blockIdx.y * d.G;
-    if (b0 >= B) return;                                          // uniform for the whole group
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int nb = min(d.G, B - b0);
-    const int i = lane & 15, kk = lane >> 4;
-    const int M = d.M;
-    const int ncols = nb * M;
-    const bool wave_on = w < d.NC;
-    const size_t total = (size_t)B * nFF;
-    const int n4max = (kFwdKC * M + 2) >> 1;                      // float4 slots of one sample's run
-    const int nslots = nb * n4max;
-
-    // the lane's two complex columns: sample, m, LDS offset of channel 0 of the stage
-    bool ok[2];
-    int col_b[2], col_m[2], lofs[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int q = w * 32 + 2 * i + h;
-        ok[h] = wave_on && q < ncols;
-        col_b[h] = ok[h] ? q / M : 0;
-        col_m[h] = ok[h] ? q - col_b[h] * M : 0;
-        const size_t soff = (size_t)(b0 + col_b[h]) * nFF + d.cumFF;   // parity is the same for every stage
-        lofs[h] = col_b[h] * 2 * n4max + (int)(soff & 1) + col_m[h];
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate); n above the table waits for all.
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define CGNET_VMCNT(N) case N: __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14)); break;
+    switch (n) {
+        CGNET_VMCNT(1) CGNET_VMCNT(2) CGNET_VMCNT(3) CGNET_VMCNT(4) CGNET_VMCNT(5) CGNET_VMCNT(6) CGNET_VMCNT(7)
+        CGNET_VMCNT(8) CGNET_VMCNT(9) CGNET_VMCNT(10) CGNET_VMCNT(11) CGNET_VMCNT(12) CGNET_VMCNT(13)
+        CGNET_VMCNT(14) CGNET_VMCNT(15) CGNET_VMCNT(16) CGNET_VMCNT(17) CGNET_VMCNT(18) CGNET_VMCNT(19)
+        CGNET_VMCNT(20) CGNET_VMCNT(21) CGNET_VMCNT(22) CGNET_VMCNT(23) CGNET_VMCNT(24) CGNET_VMCNT(25)
+        CGNET_VMCNT(26) CGNET_VMCNT(27) CGNET_VMCNT(28)
+        default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
     }
+#undef CGNET_VMCNT
+    asm volatile("" ::: "memory");
+}
 
-    float4 pre[kFwdRegs];
-    auto fetch = [&](int k0) {
+// Forward mixing.  Every wave works alone (no barrier in the kernel): it owns G whole samples
+// of one degree (G*M complex columns in T tiles of 16) and a slice of the channels, and streams
+// its samples' runs of kFwdKC channels (one contiguous run per sample) together with the
+// packed weights of those channels straight from memory into a private ring of LDS stages,
+// `depth` - 1 stages ahead of the arithmetic.  Loads complete in order, so "stage s has landed"
+// is a vmcnt wait that leaves the younger stages in flight.
+constexpr int kFwdKC = 8;        // channels per stage (two k-steps of 4)
+constexpr int kFwdMaxT = 6;      // column tiles per wave (96 complex columns)
+constexpr int kFwdDepth = 3;
+constexpr int kFwdSlice = 256;   // channels per k-slice: short enough that the groups pack the CUs evenly
+
+template <int T>
+__device__ __forceinline__ void wmm_forward_wave(const float2* __restrict__ FF, const float* __restrict__ Wp,
+                                                 float2* __restrict__ out, const WmmDeg& d, const WmmFwdUnit& u,
+                                                 int B, int nFF, int nO, int b_first, unsigned char* ring, int depth,
+                                                 int stage_bytes, int lane) {
+    const int M = d.M;
+    const int nb = min(d.G, B - b_first);
+    const int i = lane & 15, kk = lane >> 4;
+    const int run_cap = kFwdKC * M;                               // entries of one sample's run (64*M bytes)
+    bool ok[T];
+    int col_b[T], col_m[T], lofs[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const int q = 16 * t + i;
+        ok[t] = q < nb * M;
+        col_b[t] = ok[t] ? q / M : 0;
+        col_m[t] = ok[t] ? q - col_b[t] * M : 0;
+        lofs[t] = col_b[t] * run_cap + kk * M + col_m[t];        // lanes past the last column read column 0
+    }
+    {
+        // the ring starts out finite: entries a short last stage or a short last group of samples
+        // never writes are multiplied by zero weights or land in columns nobody stores
+        float4* z = reinterpret_cast<float4*>(ring);
+        for (int e = lane; e < (depth * stage_bytes) >> 4; e += 64) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    const int nk = u.k_end - u.k_begin;
+    const int nfull = nk / kFwdKC, nstages = (nk + kFwdKC - 1) / kFwdKC;
+    const int ni = 1 + nb * ((M + 15) >> 4);                      // copy instructions of a full stage
+    auto issue = [&](int s) {
+        const int k0 = u.k_begin + s * kFwdKC;
         const int n = min(kFwdKC, u.k_end - k0) * M;
-#pragma unroll
-        for (int r = 0; r < kFwdRegs; ++r) {
-            const int id = tid + r * kThreads;
-            pre[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (id < nslots) {
-                const int j = id / n4max, idx = id - j * n4max;
-                const size_t off = (size_t)(b0 + j) * nFF + d.cumFF + (size_t)k0 * M;
-                const size_t first = off & ~(size_t)1;
-                const int n4 = (n + (int)(off & 1) + 1) >> 1;
-                if (idx < n4) {
-                    if (first + 2 * (size_t)idx + 1 < total) {
-                        pre[r] = reinterpret_cast<const float4*>(FF + first)[idx];
-                    } else {
-                        const float2 z = FF[first + 2 * (size_t)idx];
-                        pre[r] = make_float4(z.x, z.y, 0.f, 0.f);
-                    }
-                }
-            }
-        }
-    };
-    auto commit = [&](float2* buf) {
-        float4* dst = reinterpret_cast<float4*>(buf);
-#pragma unroll
-        for (int r = 0; r < kFwdRegs; ++r) {
-            const int id = tid + r * kThreads;
-            if (id < nslots) dst[id] = pre[r];
-        }
-    };
-    constexpr int kSteps = kFwdKC / 4;
-    float an0[kSteps], an1[kSteps];                               // next stage's A operands
-    const size_t ap_step = (size_t)d.nrc * 128;
-    auto fetch_a = [&](int k0) {
-        const float* ap = Wp + ((size_t)(d.wp_base + ((k0 >> 2) * d.nrc + u.rc) * 2)) * 64 + lane;
-        const int steps = (min(kFwdKC, u.k_end - k0) + 3) >> 2;
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            an0[s] = an1[s] = 0.f;
-            if (s < steps) {
-                an0[s] = ap[(size_t)s * ap_step];
-                an1[s] = ap[(size_t)s * ap_step + 64];
-            }
+        unsigned char* slot = ring + (size_t)(s % depth) * stage_bytes;
+        const float* ap = Wp + (size_t)d.wp_base * 64 + ((size_t)(k0 >> 3) * d.nrc + u.rc) * 256;
+        dma16<64>(ap, slot, 64, lane);
+        for (int j = 0; j < nb; ++j) {
+            const float2* src = FF + (size_t)(b_first + j) * nFF + d.cumFF + (size_t)k0 * M;
+            unsigned char* dst = slot + 1024 + (size_t)j * run_cap * 8;
+            dma16<64>(src, dst, n >> 1, lane);
+            if (n & 1) dma8(src + (n - 1), dst + 8 * (size_t)(n - 1), lane);
         }
     };
 
-    f32x4 acc[2][4];
+    f32x4 acc[2][2 * T];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2 * T; ++t) {
         acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
         acc[1][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
-    if (u.k_begin < u.k_end) {
-        fetch(u.k_begin);
-        if (wave_on) fetch_a(u.k_begin);
-    }
-    int buf = 0;
-    for (int k0 = u.k_begin; k0 < u.k_end; k0 += kFwdKC, buf ^= 1) {
-        float2* cur = lds + (size_t)buf * stage_cap;
-        commit(cur);
-        float a0[kSteps], a1[kSteps];
+    for (int s = 0; s < min(nstages, depth - 1); ++s) issue(s);
+    for (int s = 0; s < nstages; ++s) {
+        // stages s+1 .. s+depth-2 are in flight behind stage s
+        const int youngest = min(s + depth - 2, nstages - 1);
+        wait_vmcnt(youngest < nfull ? (youngest - s) * ni : 0);
+        if (s + depth - 1 < nstages) issue(s + depth - 1);
+        const unsigned char* slot = ring + (size_t)(s % depth) * stage_bytes;
+        const float4 a = reinterpret_cast<const float4*>(slot)[lane];   // (re, im rows) of k-step 0, of k-step 1
+        const float2* cur = reinterpret_cast<const float2*>(slot + 1024);
+        // channels past the end of the degree have zero weights
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            a0[s] = an0[s];
-            a1[s] = an1[s];
-        }
-        __syncthreads();
-        if (k0 + kFwdKC < u.k_end) {
-            fetch(k0 + kFwdKC);
-            if (wave_on) fetch_a(k0 + kFwdKC);
-        }
-        if (wave_on) {
-            const int klen = min(kFwdKC, u.k_end - k0);
+        for (int q = 0; q < 2; ++q) {
+            const float a0 = q ? a.z : a.x, a1 = q ? a.w : a.y;
 #pragma unroll
-            for (int s = 0; s < kSteps; ++s) {
-                const int kl = 4 * s + kk;
-                float2 v0 = make_float2(0.f, 0.f), v1 = v0;
-                if (kl < klen) {
-                    if (ok[0]) v0 = cur[lofs[0] + kl * M];
-                    if (ok[1]) v1 = cur[lofs[1] + kl * M];
-                }
-                acc[0][0] = mfma4(a0[s], v0.x, acc[0][0]);
-                acc[0][1] = mfma4(a0[s], v0.y, acc[0][1]);
-                acc[0][2] = mfma4(a0[s], v1.x, acc[0][2]);
-                acc[0][3] = mfma4(a0[s], v1.y, acc[0][3]);
-                acc[1][0] = mfma4(a1[s], v0.x, acc[1][0]);
-                acc[1][1] = mfma4(a1[s], v0.y, acc[1][1]);
-                acc[1][2] = mfma4(a1[s], v1.x, acc[1][2]);
-                acc[1][3] = mfma4(a1[s], v1.y, acc[1][3]);
+            for (int t = 0; t < T; ++t) {
+                const float2 v = cur[lofs[t] + 4 * q * M];
+                acc[0][2 * t] = mfma4(a0, v.x, acc[0][2 * t]);
+                acc[0][2 * t + 1] = mfma4(a0, v.y, acc[0][2 * t + 1]);
+                acc[1][2 * t] = mfma4(a1, v.x, acc[1][2 * t]);
+                acc[1][2 * t + 1] = mfma4(a1, v.y, acc[1][2 * t + 1]);
             }
         }
     }
@@ -373,18 +338,50 @@ wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, 
     // complex outputs: the re / im columns of a complex column sit in the same lane
     float2* dst = out + (size_t)u.slice * B * nO;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        if (!ok[h]) continue;
+    for (int t = 0; t < T; ++t) {
+        if (!ok[t]) continue;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int to = u.rc * 16 + 4 * kk + v;
             if (to < d.tO) {
-                const float re = acc[0][2 * h][v] - acc[1][2 * h + 1][v];
-                const float im = acc[0][2 * h + 1][v] + acc[1][2 * h][v];
-                dst[(size_t)(b0 + col_b[h]) * nO + d.cumO + to * M + col_m[h]] = make_float2(re, im);
+                const float re = acc[0][2 * t][v] - acc[1][2 * t + 1][v];
+                const float im = acc[0][2 * t + 1][v] + acc[1][2 * t][v];
+                dst[(size_t)(b_first + col_b[t]) * nO + d.cumO + to * M + col_m[t]] = make_float2(re, im);
             }
         }
     }
+}
+
+// TMAX = 3 serves the degrees with up to three column tiles per wave, TMAX = 6 the others (their
+// accumulators need twice the registers).
+template <int TMAX>
+__global__ void __launch_bounds__(kThreads)
+wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
+                   const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO,
+                   int stage_bytes, int depth) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const WmmFwdUnit u = units[blockIdx.x];
+    const WmmDeg d = degs[u.deg];
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave index, held in a scalar register
+    const int b_first = (blockIdx.y * 4 + w) * d.G;
+    if (b_first >= B) return;                                     // wave-uniform; the kernel has no barrier
+    unsigned char* ring = smem + (size_t)w * depth * stage_bytes;
+#define CGNET_FWD_T(T_) wmm_forward_wave<T_>(FF, Wp, out, d, u, B, nFF, nO, b_first, ring, depth, stage_bytes, lane)
+    if (TMAX == 3) {
+        switch (d.NC) {
+            case 1: CGNET_FWD_T(1); break;
+            case 2: CGNET_FWD_T(2); break;
+            default: CGNET_FWD_T(3); break;
+        }
+    } else {
+        switch (d.NC) {
+            case 4: CGNET_FWD_T(4); break;
+            case 5: CGNET_FWD_T(5); break;
+            default: CGNET_FWD_T(6); break;
+        }
+    }
+#undef CGNET_FWD_T
 }
 
 // O = sum over k-slices of the partial outputs, in slice order
@@ -720,21 +717,21 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         d.cumFF = (int)cFF; d.cumO = (int)cO; d.cumW = (int)cW; d.cumT = (int)cT;
         d.nrc = std::max(1, (tO + 15) / 16);
         d.wp_base = wp;
-        // forward: G samples x M complex columns per wave in NC chunks of 32 columns
-        int bestG = 1, bestNC = (M + 31) / 32;
-        if (M <= 96) {
+        // forward: a wave owns G samples = G*M complex columns in NC tiles of 16 columns
+        int bestG = 1, bestNC = (M + 15) / 16;
+        {
             double best = -1;
             for (int nc = 1; nc <= 3; ++nc) {
-                const int g = (32 * nc) / M;
+                const int g = (16 * nc) / M;
                 if (g < 1) continue;
-                const double eff = (double)g * M / (32.0 * nc);
+                const double eff = (double)g * M / (16.0 * nc);
                 if (eff > best + 1e-9) { best = eff; bestG = g; bestNC = nc; }
             }
         }
         d.G = bestG;
         d.NC = bestNC;
-        // k-slices of about 768 channels (multiples of 4)
-        d.S = std::max(1, (K + 767) / 768);
+        // k-slices of about kFwdSlice channels (multiples of 8)
+        d.S = std::max(1, (K + kFwdSlice - 1) / kFwdSlice);
         d.nks_b = std::max(1, (2 * tO + 3) / 4);
         d.ap_base = p->ap_blocks;
         p->ap_blocks += ((K + 15) / 16) * d.nks_b;
@@ -744,7 +741,7 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         cO += (long long)tO * M;
         cW += (long long)K * tO;
         cT += K;
-        wp += ((K + 3) / 4) * d.nrc * 2;
+        wp += ((K + 7) / 8) * d.nrc * 4;
         CGNET_REQUIRE(cFF < (1LL << 30) && cW < (1LL << 30), CGNET_ERR_UNSUPPORTED, "sizes above 2^30 complex entries");
     }
     p->nFF = (int)cFF; p->nO = (int)cO; p->nW = (int)cW; p->sumT = (int)cT;
@@ -753,12 +750,12 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
     for (int di = 0; di < ndeg; ++di) {
         const WmmDeg& d = p->degs[di];
         if (d.K == 0 || d.tO == 0) continue;
-        CGNET_REQUIRE(d.NC <= 3, CGNET_ERR_UNSUPPORTED, "degree %d has more than 96 columns per sample", d.l);
+        CGNET_REQUIRE(d.NC <= kFwdMaxT, CGNET_ERR_UNSUPPORTED, "degree %d has more than 96 columns per sample", d.l);
         p->maxS = std::max(p->maxS, d.S);
         p->maxG = std::max(p->maxG, d.G);
-        p->fwd_stage_cap = std::max(p->fwd_stage_cap, d.G * 2 * ((kFwdKC * d.M + 2) / 2));
-        const int steps = (d.K + 3) / 4;
-        const int per = ((steps + d.S - 1) / d.S) * 4;
+        p->fwd_stage_cap = std::max(p->fwd_stage_cap, 1024 + d.G * kFwdKC * d.M * 8);   // bytes: weights + runs
+        const int steps = (d.K + 7) / 8;
+        const int per = ((steps + d.S - 1) / d.S) * 8;
         for (int rc = 0; rc < d.nrc; ++rc)
             for (int s = 0; s < d.S; ++s) {
                 WmmFwdUnit u{di, rc, s, std::min(d.K, s * per), std::min(d.K, (s + 1) * per)};
@@ -808,6 +805,18 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
     };
     int rc;
     if ((rc = upload(p->degs.data(), sizeof(WmmDeg) * ndeg, (void**)&p->d_degs))) return rc;
+    {
+        // longest units first, so that the last groups to start are short ones
+        auto work = [&](const WmmFwdUnit& u) {
+            const WmmDeg& d = p->degs[u.deg];
+            return (long long)(u.k_end - u.k_begin) * d.M * d.G;
+        };
+        std::stable_sort(p->fwd_units.begin(), p->fwd_units.end(),
+                         [&](const WmmFwdUnit& a, const WmmFwdUnit& b) { return work(a) > work(b); });
+        auto mid = std::stable_partition(p->fwd_units.begin(), p->fwd_units.end(),
+                                         [&](const WmmFwdUnit& u) { return p->degs[u.deg].NC <= 3; });
+        p->fwd_units_small = (int)(mid - p->fwd_units.begin());
+    }
     if ((rc = upload(p->fwd_units.data(), sizeof(WmmFwdUnit) * p->fwd_units.size(), (void**)&p->d_fwd_units))) return rc;
     if ((rc = upload(p->gw_units.data(), sizeof(WmmChanUnit) * p->gw_units.size(), (void**)&p->d_gw_units))) return rc;
     for (const WmmChanUnit& u : p->gw_units)
@@ -905,13 +914,24 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     }
     int ygroups = 1;
     for (const WmmDeg& d : plan->degs)
-        if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + d.G - 1) / d.G);
+        if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + 4 * d.G - 1) / (4 * d.G));
     CGNET_REQUIRE(ygroups <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d too large", B);
-    CGNET_REQUIRE(((uintptr_t)d_FF & 15) == 0, CGNET_ERR_ARG, "d_FF must be 16-byte aligned");
-    CGNET_LAUNCH(wmm_forward_kernel, dim3((unsigned)plan->fwd_units.size(), ygroups), dim3(kThreads),
-                 sizeof(float2) * 2 * (size_t)plan->fwd_stage_cap, s, (const float2*)d_FF, Wp, out, plan->d_degs,
-                 plan->d_fwd_units, B, plan->nFF, plan->nO, plan->fwd_stage_cap);
-    CGNET_HIP(hipGetLastError());
+    // the LDS-direct copies address the first 64 KB of a group's LDS
+    const int depth = (int)std::min<size_t>(kFwdDepth, (64 * 1024) / (4 * (size_t)plan->fwd_stage_cap));
+    CGNET_REQUIRE(depth >= 2, CGNET_ERR_UNSUPPORTED, "forward stage of %d bytes does not fit the LDS ring", plan->fwd_stage_cap);
+    const size_t lds = 4 * (size_t)depth * plan->fwd_stage_cap;
+    if (plan->fwd_units_small > 0) {
+        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3((unsigned)plan->fwd_units_small, ygroups), dim3(kThreads), lds, s,
+                     (const float2*)d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO,
+                     plan->fwd_stage_cap, depth);
+        CGNET_HIP(hipGetLastError());
+    }
+    if ((int)plan->fwd_units.size() > plan->fwd_units_small) {
+        CGNET_LAUNCH(wmm_forward_kernel<6>, dim3((unsigned)(plan->fwd_units.size() - plan->fwd_units_small), ygroups),
+                     dim3(kThreads), lds, s, (const float2*)d_FF, Wp, out, plan->d_degs,
+                     plan->d_fwd_units + plan->fwd_units_small, B, plan->nFF, plan->nO, plan->fwd_stage_cap, depth);
+        CGNET_HIP(hipGetLastError());
+    }
     if (plan->maxS > 1) {
         const size_t n = (size_t)plan->nO * B;
         CGNET_LAUNCH(wmm_sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
