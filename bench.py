@@ -73,6 +73,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-repeats", type=int, default=2)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 768 MiB read + 768 MiB write elementwise kernel before the warm-up "
+                         "(a known-size reference for calibrating hardware byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs the CG layer on ONE GPU (no collectives, no sharding); "
@@ -104,6 +107,13 @@ def main():
         out = layer(x, straight_output=True)
         out.backward(go)
 
+    if args.copy_probe:
+        src = torch.ones(192 * 1024 * 1024, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -134,6 +144,12 @@ def main():
         "cg_backward_unit_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
+    # HBM bytes per launch at this workload from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
+    # profiles/cg_layer_L11_tau12_B100_hbm_traffic_pmc.txt (calibrated against a copy kernel of known size)
+    measured_traffic = {
+        "cg_backward_unit_kernel": 840.1e6, "cg_forward_kernel": 794.5e6, "wmm_forward_kernel": 926.5e6,
+        "wmm_gradw_kernel": 808.2e6, "wmm_gradff_mfma_kernel": 833.4e6,
+    }
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
     kernels = {}
     for name, (ms, cnt) in sorted(times.items(), key=lambda kv: -kv[1][0]):
@@ -159,7 +175,7 @@ def main():
                                "CG product + fragment norm + weight mixing, default (l2<=l1) triples",
                    "lmax": lmax, "tau": tau, "batch": bsz, "triples": len(layer.cg.lll_list)},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic.get(dominant),
                      "algorithmic_bytes_per_launch": algo[dominant], "avg_launch_ms": d_avg_s * 1e3},
         "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
                        "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
