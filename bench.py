@@ -71,8 +71,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-batch", type=int, default=8)
-    ap.add_argument("--cpu-repeats", type=int, default=2)
+    ap.add_argument("--cpu-batch", type=int, default=16)
+    ap.add_argument("--cpu-repeats", type=int, default=6)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 768 MiB read + 768 MiB write elementwise kernel before the warm-up "
                          "(a known-size reference for calibrating hardware byte counters)")
