@@ -51,7 +51,7 @@ struct cgnet_wmm_plan {
     bool gff_mfma = true;  // every degree has t_O <= 16 (the operand then fits eight registers)
     int gw_ff_cap = 2, gw_go_cap = 2;   // LDS capacities (complex entries) of one stage of the weight-gradient kernel
     int fwd_stage_cap = 16;             // LDS bytes of one stage of one wave of the forward kernel
-    int gff_out_cap = 4, gff_go_cap = 2; // LDS capacities of the FF-gradient kernel (real entries / complex entries)
+    int gff_out_cap = 16, gff_go_cap = 16; // LDS bytes per wave of the FF-gradient kernel: result tile / one gO buffer
     int maxS = 1, maxG = 1;
     std::vector<cgnet::WmmDeg> degs;
     std::vector<cgnet::WmmFwdUnit> fwd_units;   // units of degrees with NC <= 3 first
@@ -578,83 +578,121 @@ pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ std
     Ap[idx] = v;
 }
 
-constexpr int kGffGORegs = 3;   // float4 registers per thread for the gO rows of one sample (t_O <= 16 rows)
+// Gradient with respect to FF on the matrix cores (t_O <= 16): gFF[c, (m, re/im)] = sum_k A[c, k] * B[k, (m, re/im)]
+// with k = (to, re/im).  Every wave works alone (no barrier): it owns 16 channels of the unit and
+// walks over the samples of its group.  The gO rows of the next sample arrive by LDS-direct loads
+// while the current one is multiplied; the 16 x 2M result tile goes through the wave's LDS image
+// and leaves as one contiguous run of 16-byte stores, one sample behind the arithmetic, so the
+// wait for the next operands never waits for fresh stores.
+template <int NKS>
+__device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, const float* __restrict__ Ap,
+                                                float2* __restrict__ gFF, const WmmDeg& d, const WmmChanUnit& u, int B,
+                                                int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes,
+                                                unsigned char* mine, int w, int lane) {
+    float* ol = reinterpret_cast<float*>(mine);                              // [16][2M]
+    unsigned char* gobuf = mine + out_bytes;                                  // [2][go_bytes]
+    const int i = lane & 15, kk = lane >> 4;
+    const int M = d.M, tO = d.tO;
+    constexpr int nks = NKS;
+    const int ctile = (u.c0 >> 4) + w;
+    float a[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) a[ks] = Ap[((size_t)d.ap_base + (size_t)ctile * nks + ks) * 64 + lane];
+    // k = 4*ks + kk  ->  to = 2*ks + (kk >> 1), re/im = kk & 1;  column 16*ct + i -> m = 8*ct + (i >> 1), re/im = i & 1
+    const int to_lane = kk >> 1, sel = kk & 1, r = i & 1;
+    const float cx = (r == sel) ? (r ? -1.f : 1.f) : 0.f, cy = (r == sel) ? 0.f : 1.f;   // B = cx * re + cy * im
+    const int nct = (2 * M + 15) >> 4;
+    const int rows = min(16, u.nc - 16 * w);
+    const int n_go = tO * M, n_out = rows * M;    // complex entries of the gO rows / of this wave's output run
+    const int b_begin = blockIdx.y * samples_per_group, b_end = min(B, b_begin + samples_per_group);
+    if (b_begin >= b_end) return;
+    {
+        // rows past t_O are read (times zero weights): they must hold finite values
+        float4* z = reinterpret_cast<float4*>(gobuf);
+        for (int e = lane; e < (2 * go_bytes) >> 4; e += 64) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    auto issue = [&](int b, int par) {
+        const float2* src = gO + (size_t)b * nO + d.cumO;
+        unsigned char* dst = gobuf + (size_t)par * go_bytes;
+        dma16<64>(src, dst, n_go >> 1, lane);
+        if (n_go & 1) dma8(src + (n_go - 1), dst + 8 * (size_t)(n_go - 1), lane);
+    };
+    auto store_tile = [&](int b) {
+        const size_t off = (size_t)b * nFF + d.cumFF + (size_t)(u.c0 + 16 * w) * M;
+        float2* dst = gFF + off;
+        const float2* src = reinterpret_cast<const float2*>(ol);
+        const int head = (int)(off & 1);          // unaligned first entry
+        if (head && lane == 0) dst[0] = src[0];
+        const int n4 = (n_out - head) >> 1;
+        for (int idx = lane; idx < n4; idx += 64) {
+            const float2 z0 = src[head + 2 * idx], z1 = src[head + 2 * idx + 1];
+            *reinterpret_cast<float4*>(dst + head + 2 * idx) = make_float4(z0.x, z0.y, z1.x, z1.y);
+        }
+        if (((n_out - head) & 1) && lane == 0) dst[n_out - 1] = src[n_out - 1];
+    };
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the clearing stores precede the first copy
+    issue(b_begin, 0);
+    const int row0 = 4 * kk;                      // D rows of this lane inside the wave's tile
+    int par = 0;
+    for (int b = b_begin; b < b_end; ++b, par ^= 1) {
+        dma_wait();                               // gO rows of sample b are in LDS
+        asm volatile("" ::: "memory");
+        if (b > b_begin) store_tile(b - 1);
+        if (b + 1 < b_end) issue(b + 1, par ^ 1);
+        const float2* g = reinterpret_cast<const float2*>(gobuf + (size_t)par * go_bytes);
+        for (int ct0 = 0; ct0 < nct; ct0 += 3) {
+            f32x4 acc[3];
+            int mofs[3];
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                mofs[t] = min(8 * (ct0 + t) + (i >> 1), M - 1);           // clamped: extra columns are not stored
+            }
+            float bv[NKS][3];
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int to = min(2 * ks + to_lane, tO - 1);             // clamped: rows past t_O carry zero weights
+#pragma unroll
+                for (int t = 0; t < 3; ++t) {
+                    const float2 z = g[to * M + mofs[t]];
+                    bv[ks][t] = fmaf(z.x, cx, z.y * cy);
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+                for (int t = 0; t < 3; ++t) acc[t] = mfma4(a[ks], bv[ks][t], acc[t]);
+            mfma_drain();
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                const int col = (ct0 + t) * 16 + i;
+                if (col < 2 * M) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) ol[(size_t)(row0 + v) * 2 * M + col] = acc[t][v];
+                }
+            }
+        }
+    }
+    store_tile(b_end - 1);
+}
 
 __global__ void __launch_bounds__(kThreads)
 wmm_gradff_mfma_kernel(const float2* __restrict__ gO, const float* __restrict__ Ap, float2* __restrict__ gFF,
                        const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
-                       int samples_per_group, int nFF, int nO, int out_cap, int go_cap) {
+                       int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* outbuf = reinterpret_cast<float*>(smem);                          // [2][out_cap] real entries
-    float2* gobuf = reinterpret_cast<float2*>(outbuf + 2 * (size_t)out_cap);  // [2][go_cap]
     const WmmChanUnit u = units[blockIdx.x];
     const WmmDeg d = degs[u.deg];
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const bool wave_on = 16 * w < u.nc;
-    const int i = lane & 15, kk = lane >> 4;
-    const int M = d.M, tO = d.tO, nks = d.nks_b;
-    const int ctile = (u.c0 >> 4) + w;
-    float a[8];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-        a[ks] = (wave_on && ks < nks) ? Ap[((size_t)d.ap_base + (size_t)ctile * nks + ks) * 64 + lane] : 0.f;
-    const int to_lane = kk >> 1, sel = kk & 1;   // k = 4*ks + kk  ->  to = 2*ks + to_lane, re/im = sel
-    const int nct = (2 * M + 15) >> 4;
-    const int row0 = 16 * w + 4 * kk;            // D rows of this lane inside the group's tile
-    const int n_go = tO * M, n_out = u.nc * M;   // complex entries of the gO rows / of the output run
-    const size_t tot_go = (size_t)B * nO;
-    const int b_begin = blockIdx.y * samples_per_group, b_end = min(B, b_begin + samples_per_group);
-    auto go_off = [&](int b) { return (size_t)b * nO + d.cumO; };
-
-    Run16<kGffGORegs> pg;
-    if (b_begin < b_end) pg.fetch(gO, go_off(b_begin), n_go, tot_go, tid, kThreads);
-    int buf = 0;
-    for (int b = b_begin; b < b_end; ++b, buf ^= 1) {
-        float* ol = outbuf + (size_t)buf * out_cap;
-        float2* gl = gobuf + (size_t)buf * go_cap;
-        const size_t go_ = go_off(b);
-        pg.commit(gl, go_, n_go, tid, kThreads);
-        __syncthreads();                          // gO rows of sample b visible; tile buffer `buf` is free again
-        if (b + 1 < b_end) pg.fetch(gO, go_off(b + 1), n_go, tot_go, tid, kThreads);
-        if (wave_on) {
-            const float2* g = gl + (go_ & 1);
-            for (int ct = 0; ct < nct; ++ct) {
-                const int col = ct * 16 + i;
-                const int m = col >> 1, r = col & 1;
-                const bool cok = m < M;
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < 8; ++ks) {
-                    if (ks < nks) {
-                        float bv = 0.f;
-                        const int to = 2 * ks + to_lane;
-                        if (cok && to < tO) {
-                            const float2 z = g[to * M + m];
-                            bv = (r == sel) ? (r ? -z.x : z.x) : z.y;
-                        }
-                        acc = mfma4(a[ks], bv, acc);
-                    }
-                }
-                mfma_drain();
-                if (cok) {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) ol[(size_t)(row0 + v) * 2 * M + col] = acc[v];
-                }
-            }
-        }
-        __syncthreads();                          // the tile of sample b is complete
-        // stream the tile out: one contiguous run of n_out complex numbers
-        float2* dst = gFF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M;
-        const float2* src = reinterpret_cast<const float2*>(ol);
-        const int head = (int)(((size_t)b * nFF + d.cumFF + (size_t)u.c0 * M) & 1);   // unaligned first entry
-        if (head && tid == 0 && n_out > 0) dst[0] = src[0];
-        const int n4 = (n_out - head) >> 1;
-        for (int idx = tid; idx < n4; idx += kThreads) {
-            const float2 z0 = src[head + 2 * idx], z1 = src[head + 2 * idx + 1];
-            *reinterpret_cast<float4*>(dst + head + 2 * idx) = make_float4(z0.x, z0.y, z1.x, z1.y);
-        }
-        if (((n_out - head) & 1) && tid == 0) dst[n_out - 1] = src[n_out - 1];
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (16 * w >= u.nc) return;                   // wave-uniform; the kernel has no barrier
+    unsigned char* mine = smem + (size_t)w * (out_bytes + 2 * go_bytes);
+#define CGNET_GFF(N_) case N_: wmm_gradff_wave<N_>(gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane); break;
+    switch (d.nks_b) {
+        CGNET_GFF(1) CGNET_GFF(2) CGNET_GFF(3) CGNET_GFF(4) CGNET_GFF(5) CGNET_GFF(6) CGNET_GFF(7)
+        default: wmm_gradff_wave<8>(gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane); break;
     }
+#undef CGNET_GFF
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(float* p, size_t n) {
@@ -766,8 +804,8 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         for (int rc = 0; rc < d.nrc; ++rc)
             for (int c0 = 0; c0 < d.K; c0 += gw_nc)
                 p->gw_units.push_back(WmmChanUnit{di, rc, c0, std::min(gw_nc, d.K - c0)});
-        p->gff_out_cap = std::max(p->gff_out_cap, (int)align_up((size_t)gw_nc * d.M * 2, 4));
-        p->gff_go_cap = std::max(p->gff_go_cap, (int)align_up((size_t)std::min(d.tO, 16) * d.M + 2, 2));
+        p->gff_out_cap = std::max(p->gff_out_cap, (int)align_up((size_t)16 * d.M * 8, 16));                       // bytes per wave
+        p->gff_go_cap = std::max(p->gff_go_cap, (int)align_up((size_t)std::min(d.tO, 16) * d.M * 8 + 16, 16));   // bytes per wave and buffer
         p->gw_ff_cap = std::max(p->gw_ff_cap, (int)align_up((size_t)gw_nc * d.M + 2, 2));
         p->gw_go_cap = std::max(p->gw_go_cap, (int)align_up((size_t)16 * d.M + 2, 2));
     }
@@ -783,6 +821,8 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
             p->gff_units.push_back(WmmChanUnit{di, 0, c0, std::min(per_gff, d.K - c0)});
         p->gff_lds = std::max(p->gff_lds, (size_t)8 * d.tO * d.M);
     }
+    // the matrix-core gradient kernel keeps a tile and two operand buffers per wave inside 64 KB of LDS
+    if (4 * ((size_t)p->gff_out_cap + 2 * (size_t)p->gff_go_cap) > 64 * 1024) p->gff_mfma = false;
     CGNET_REQUIRE(p->gff_lds <= 64 * 1024, CGNET_ERR_UNSUPPORTED, "t_O*(2l+1) too large for the gradient kernel");
     // heavier forward units first
     std::stable_sort(p->fwd_units.begin(), p->fwd_units.end(), [&](const WmmFwdUnit& a, const WmmFwdUnit& b) {
@@ -1001,10 +1041,11 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_HIP(hipGetLastError());
             const int groups = std::max(1, std::min(B, 8));
             const int spg = (B + groups - 1) / groups;
-            const size_t lds = 2 * (sizeof(float) * (size_t)plan->gff_out_cap + sizeof(float2) * (size_t)plan->gff_go_cap);
+            const int out_bytes = plan->gff_out_cap, go_bytes = plan->gff_go_cap;   // per wave
+            const size_t lds = 4 * ((size_t)out_bytes + 2 * (size_t)go_bytes);
             CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)plan->gw_units_rc0.size(), (B + spg - 1) / spg),
                          dim3(kThreads), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
-                         plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, plan->gff_out_cap, plan->gff_go_cap);
+                         plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, out_bytes, go_bytes);
             CGNET_HIP(hipGetLastError());
         } else {
             if (plan->nW > 0) {
