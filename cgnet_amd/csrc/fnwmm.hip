@@ -584,7 +584,8 @@ pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ std
 // while the current one is multiplied; the 16 x 2M result tile goes through the wave's LDS image
 // and leaves as one contiguous run of 16-byte stores, one sample behind the arithmetic, so the
 // wait for the next operands never waits for fresh stores.
-template <int NKS>
+// NT = column tiles worked on together (all of them when the degree has at most three)
+template <int NKS, int NT>
 __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, const float* __restrict__ Ap,
                                                 float2* __restrict__ gFF, const WmmDeg& d, const WmmChanUnit& u, int B,
                                                 int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes,
@@ -640,20 +641,20 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
         if (b > b_begin) store_tile(b - 1);
         if (b + 1 < b_end) issue(b + 1, par ^ 1);
         const float2* g = reinterpret_cast<const float2*>(gobuf + (size_t)par * go_bytes);
-        for (int ct0 = 0; ct0 < nct; ct0 += 3) {
-            f32x4 acc[3];
-            int mofs[3];
+        for (int ct0 = 0; ct0 < nct; ct0 += NT) {
+            f32x4 acc[NT];
+            int mofs[NT];
 #pragma unroll
-            for (int t = 0; t < 3; ++t) {
+            for (int t = 0; t < NT; ++t) {
                 acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 mofs[t] = min(8 * (ct0 + t) + (i >> 1), M - 1);           // clamped: extra columns are not stored
             }
-            float bv[NKS][3];
+            float bv[NKS][NT];
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 const int to = min(2 * ks + to_lane, tO - 1);             // clamped: rows past t_O carry zero weights
 #pragma unroll
-                for (int t = 0; t < 3; ++t) {
+                for (int t = 0; t < NT; ++t) {
                     const float2 z = g[to * M + mofs[t]];
                     bv[ks][t] = fmaf(z.x, cx, z.y * cy);
                 }
@@ -661,10 +662,10 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-                for (int t = 0; t < 3; ++t) acc[t] = mfma4(a[ks], bv[ks][t], acc[t]);
+                for (int t = 0; t < NT; ++t) acc[t] = mfma4(a[ks], bv[ks][t], acc[t]);
             mfma_drain();
 #pragma unroll
-            for (int t = 0; t < 3; ++t) {
+            for (int t = 0; t < NT; ++t) {
                 const int col = (ct0 + t) * 16 + i;
                 if (col < 2 * M) {
 #pragma unroll
@@ -687,11 +688,23 @@ wmm_gradff_mfma_kernel(const float2* __restrict__ gO, const float* __restrict__ 
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (16 * w >= u.nc) return;                   // wave-uniform; the kernel has no barrier
     unsigned char* mine = smem + (size_t)w * (out_bytes + 2 * go_bytes);
-#define CGNET_GFF(N_) case N_: wmm_gradff_wave<N_>(gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane); break;
+#define CGNET_GFF_ARGS gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane
+#define CGNET_GFF(N_)                                                                     \
+    case N_:                                                                              \
+        if (nct == 1) wmm_gradff_wave<N_, 1>(CGNET_GFF_ARGS);                             \
+        else if (nct == 2) wmm_gradff_wave<N_, 2>(CGNET_GFF_ARGS);                        \
+        else wmm_gradff_wave<N_, 3>(CGNET_GFF_ARGS);                                      \
+        break;
+    const int nct = (2 * d.M + 15) >> 4;
     switch (d.nks_b) {
         CGNET_GFF(1) CGNET_GFF(2) CGNET_GFF(3) CGNET_GFF(4) CGNET_GFF(5) CGNET_GFF(6) CGNET_GFF(7)
-        default: wmm_gradff_wave<8>(gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane); break;
+        default:
+            if (nct == 1) wmm_gradff_wave<8, 1>(CGNET_GFF_ARGS);
+            else if (nct == 2) wmm_gradff_wave<8, 2>(CGNET_GFF_ARGS);
+            else wmm_gradff_wave<8, 3>(CGNET_GFF_ARGS);
+            break;
     }
+#undef CGNET_GFF_ARGS
 #undef CGNET_GFF
 }
 
