@@ -290,18 +290,40 @@ __device__ __forceinline__ void wmm_forward_wave(const float2* __restrict__ FF, 
     }
     const int nk = u.k_end - u.k_begin;
     const int nfull = nk / kFwdKC, nstages = (nk + kFwdKC - 1) / kFwdKC;
-    const int ni = 1 + nb * ((M + 15) >> 4);                      // copy instructions of a full stage
-    auto issue = [&](int s) {
-        const int k0 = u.k_begin + s * kFwdKC;
-        const int n = min(kFwdKC, u.k_end - k0) * M;
-        unsigned char* slot = ring + (size_t)(s % depth) * stage_bytes;
-        const float* ap = Wp + (size_t)d.wp_base * 64 + ((size_t)(k0 >> 3) * d.nrc + u.rc) * 256;
-        dma16<64>(ap, slot, 64, lane);
-        for (int j = 0; j < nb; ++j) {
-            const float2* src = FF + (size_t)(b_first + j) * nFF + d.cumFF + (size_t)k0 * M;
-            unsigned char* dst = slot + 1024 + (size_t)j * run_cap * 8;
-            dma16<64>(src, dst, n >> 1, lane);
-            if (n & 1) dma8(src + (n - 1), dst + 8 * (size_t)(n - 1), lane);
+    // A full stage is one list of 16-byte pieces, sample after sample (4*M pieces per run), that
+    // lands contiguously behind the weights: piece c = lane + 64*r comes from a per-lane address
+    // fixed for the whole slice plus the stage's offset.
+    const int cpr = 4 * M, npieces = nb * cpr;
+    const int nr = (npieces + 63) >> 6;                           // <= T copy instructions per stage
+    const int ni = 1 + nr;                                        // copy instructions of a full stage
+    const char* piece[T];
+#pragma unroll
+    for (int r = 0; r < T; ++r) {
+        const int c = min(lane + 64 * r, npieces - 1);
+        const int j = c / cpr, idx = c - j * cpr;
+        piece[r] = reinterpret_cast<const char*>(FF + (size_t)(b_first + j) * nFF + d.cumFF + (size_t)u.k_begin * M) + 16 * idx;
+    }
+    const char* wpiece = reinterpret_cast<const char*>(Wp + (size_t)d.wp_base * 64 +
+                                                       ((size_t)(u.k_begin >> 3) * d.nrc + u.rc) * 256) + 16 * lane;
+    const size_t w_step = (size_t)d.nrc * 1024, f_step = (size_t)kFwdKC * M * 8;
+    auto issue = [&](int s, int slot_idx) {
+        unsigned char* slot = ring + (size_t)slot_idx * stage_bytes;
+        __builtin_amdgcn_global_load_lds(wpiece + (size_t)s * w_step, (lds_void_ptr)slot, 16, 0, 0);
+        if (s < nfull) {
+#pragma unroll
+            for (int r = 0; r < T; ++r)
+                if (r < nr && lane + 64 * r < npieces)
+                    __builtin_amdgcn_global_load_lds(piece[r] + (size_t)s * f_step, (lds_void_ptr)(slot + 1024 + 1024 * r), 16, 0, 0);
+        } else {
+            // the short last stage of a degree whose channel count is no multiple of kFwdKC
+            const int k0 = u.k_begin + s * kFwdKC;
+            const int n = (u.k_end - k0) * M;
+            for (int j = 0; j < nb; ++j) {
+                const float2* src = FF + (size_t)(b_first + j) * nFF + d.cumFF + (size_t)k0 * M;
+                unsigned char* dst = slot + 1024 + (size_t)j * run_cap * 8;
+                dma16<64>(src, dst, n >> 1, lane);
+                if (n & 1) dma8(src + (n - 1), dst + 8 * (size_t)(n - 1), lane);
+            }
         }
     };
 
@@ -311,13 +333,16 @@ __device__ __forceinline__ void wmm_forward_wave(const float2* __restrict__ FF, 
         acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
         acc[1][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
-    for (int s = 0; s < min(nstages, depth - 1); ++s) issue(s);
+    for (int s = 0; s < min(nstages, depth - 1); ++s) issue(s, s);
+    int cur_slot = 0, next_slot = (depth - 1) % depth;            // ring positions of stage s and of stage s+depth-1
     for (int s = 0; s < nstages; ++s) {
         // stages s+1 .. s+depth-2 are in flight behind stage s
         const int youngest = min(s + depth - 2, nstages - 1);
         wait_vmcnt(youngest < nfull ? (youngest - s) * ni : 0);
-        if (s + depth - 1 < nstages) issue(s + depth - 1);
-        const unsigned char* slot = ring + (size_t)(s % depth) * stage_bytes;
+        if (s + depth - 1 < nstages) issue(s + depth - 1, next_slot);
+        const unsigned char* slot = ring + (size_t)cur_slot * stage_bytes;
+        cur_slot = cur_slot + 1 == depth ? 0 : cur_slot + 1;
+        next_slot = next_slot + 1 == depth ? 0 : next_slot + 1;
         const float4 a = reinterpret_cast<const float4*>(slot)[lane];   // (re, im rows) of k-step 0, of k-step 1
         const float2* cur = reinterpret_cast<const float2*>(slot + 1024);
         // channels past the end of the degree have zero weights
@@ -383,6 +408,11 @@ wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, 
     }
 #undef CGNET_FWD_T
 }
+
+template __global__ void wmm_forward_kernel<3>(const float2*, const float*, float2*, const WmmDeg*, const WmmFwdUnit*, int,
+                                               int, int, int, int);
+template __global__ void wmm_forward_kernel<6>(const float2*, const float*, float2*, const WmmDeg*, const WmmFwdUnit*, int,
+                                               int, int, int, int);
 
 // O = sum over k-slices of the partial outputs, in slice order
 __global__ void __launch_bounds__(256)
