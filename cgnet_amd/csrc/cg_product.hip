@@ -554,6 +554,16 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 
 // ---- register-resident backward ------------------------------------------------------------
 struct BwdGeom { int l, l1, l2, rows, tau2; };
+
+// Item -> (window of two m, first output channel).  Windows are numbered from the middle of the m
+// axis outwards and the channel groups of one window are neighbours, so the lanes of a wave have
+// similar numbers of terms and the waves with the short (outer) windows finish early.
+__device__ __forceinline__ void bwd_item(int item, int nT, int nWin, int& w, int& to) {
+    const int widx = item / nT;
+    to = item - widx * nT;
+    const int c = (nWin - 1) >> 1;
+    w = (widx & 1) ? c + ((widx + 1) >> 1) : c - (widx >> 1);
+}
 constexpr int kBwdMaxTI = 4;   // output channels per thread
 // Zero rows before / after the staged CG table.  The two m outputs of a thread and the two-step
 // unrolled loop touch table rows -1 .. M+1; there the coefficient is zero, so whatever finite
@@ -581,7 +591,8 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     const int nT = (n_o + TI - 1) / TI;
     const int nWin = (M_o + 1) >> 1;
     if (item >= nT * nWin) return;
-    const int w = item % nWin, to = item / nWin;
+    int w, to;
+    bwd_item(item, nT, nWin, w, to);
     const int mo0 = 2 * w;
     const int ir_lo = max(0, d - mo0 - 1);
     const int ir_hi = min(M_r - 1, M - 1 + d - mo0);
@@ -679,7 +690,8 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
     const int nT = (n_o + TI - 1) / TI;
     const int nWin = (M_o + 1) >> 1;
     if (item < nT * nWin) {
-        const int w = item % nWin, to = item / nWin;
+        int w, to;
+        bwd_item(item, nT, nWin, w, to);
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             const int mo = 2 * w + k;
