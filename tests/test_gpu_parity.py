@@ -457,6 +457,71 @@ def test_full_size_layer_config3_runs(dev):
     assert torch.allclose(mod.bnWMM.bn_stds, mod2.bnWMM.bn_stds, rtol=1e-6, atol=1e-9)
 
 
+@pytest.mark.parametrize("sparse", [True, False])
+def test_full_size_properties_config4(dev, sparse):
+    """BASELINE config 4 (L=15, tau=16, B=64, MST and default triples): CG product forward + backward."""
+    from cgnet_amd import CG_layers
+    lmax, taus, bsz = 15, [16] * 16, 64
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, lll_mode="mst" if sparse else None, device=dev)
+    x = rand_straight(taus, bsz, 21).float().to(dev)
+    y = mod(x)
+    assert y.shape[0] == bsz and torch.isfinite(y).all()
+    assert torch.allclose(mod(2 * x), 4 * y, rtol=1e-6, atol=1e-7)                  # bilinear
+    y5 = mod(x[5:6].contiguous())
+    assert torch.equal(y5[0], y[5])                                               # samples independent
+    # against the oracle on one sample (the CPU restatement needs seconds for one sample of this size)
+    want, _ = cg_oracle_fwd_bwd(lmax, taus, mod.lll_list, x[5:6].double().cpu())
+    assert_close(y5, want, "config 4 forward, one sample")
+    # adjoint identity of the bilinear map
+    dx = 1e-2 * torch.randn_like(x)
+    gy = torch.randn_like(y)
+    xr = x.clone().requires_grad_(True)
+    mod(xr).backward(gy)
+    assert torch.isfinite(xr.grad).all()
+    jdx = (mod(x + dx) - y - mod(dx)).double()
+    lhs = float((gy.double() * jdx).sum())
+    rhs = float((xr.grad.double() * dx.double()).sum())
+    assert lhs == pytest.approx(rhs, rel=2e-4)
+
+
+def test_full_size_stack_config5_runs(dev):
+    """BASELINE config 5 (L=20, taus 1 -> 16 x 4, B=32): SphericalCNN embedding, linear head, cross-entropy."""
+    from cgnet_amd import CGNet
+    lmax, bsz = 20, 32
+    taus = [[1] * 21] + [[16] * 21] * 4
+    net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
+    assert net.output_length == 2 * (1 + 4 * 16)
+    g = torch.Generator().manual_seed(5)
+    x = rand_straight(taus[0], bsz, 5).float()
+    head = torch.nn.Linear(net.output_length, 10).to(dev)
+    labels = torch.randint(0, 10, (bsz,), generator=g).to(dev)
+    x = x.to(dev).requires_grad_(True)
+    net.train()
+    emb = net(x)
+    assert emb.shape == (bsz, net.output_length) and torch.isfinite(emb).all()
+    loss = torch.nn.functional.cross_entropy(head(emb), labels)
+    loss.backward()
+    assert torch.isfinite(x.grad).all()
+    for cg in net.cgs:
+        assert torch.isfinite(cg.bnWMM.W.grad).all() and float(cg.bnWMM.W.grad.abs().max()) > 0
+        assert cg.bnWMM.bn_cnt == 2.0
+    # directional derivative of the loss along a random input direction, evaluation mode (fixed statistics)
+    net.eval()
+    x0 = x.detach()
+    d = torch.randn_like(x0)
+    d /= d.norm()
+
+    def f(t):
+        with torch.no_grad():
+            return float(torch.nn.functional.cross_entropy(head(net(t)).double(), labels))
+    xe = x0.clone().requires_grad_(True)
+    torch.nn.functional.cross_entropy(head(net(xe)), labels).backward()
+    want = float((xe.grad.double() * d.double()).sum())
+    h = 1e-2
+    got = (f(x0 + h * d) - f(x0 - h * d)) / (2 * h)
+    assert got == pytest.approx(want, rel=5e-2, abs=1e-5)
+
+
 # ------------------------------------------------------------------------------- error behaviour
 def test_errors(dev):
     from cgnet_amd import CG_cuda_ops, CG_layers, _plans
