@@ -137,78 +137,91 @@ __device__ __forceinline__ float sqrt_refined(float n) {
 }
 
 // One item = one m of a TI x TJ tile of channels.  Items are ordered m-major, so the lanes of a
-// wave work on neighbouring m (similar numbers of terms) of all channel tiles.
+// wave work on neighbouring m (similar numbers of terms) of all channel tiles.  What an item needs
+// to know does not depend on the sample: it is worked out once per group.
 template <int TI, int TJ>
-__device__ __forceinline__ void fwd_tiles(const CgTask& t, const float* __restrict__ cg,
-                                          const float2* __restrict__ f1, const float2* __restrict__ f2,
-                                          float2* __restrict__ out) {
+struct FwdItem {
+    unsigned pa[TI], pb[TJ];   // LDS byte addresses in fragment buffer 0: slot-1 rows (walked down), slot-2 rows (up)
+    unsigned pc, pc_end;       // table entries of the first / last term
+    int obase;                 // index in the output tile of (first channel of the tile, m)
+    int valid;                 // bit i*TJ+j: channel (i, j) of the tile exists
+    bool any;                  // the m has at least one term
+};
+
+template <int TI, int TJ>
+__device__ __forceinline__ void fwd_item_setup(const CgTask& t, int item, const float* cg, const float2* f1,
+                                               const float2* f2, FwdItem<TI, TJ>& it) {
     const int l = t.l, l1 = t.l1, l2 = t.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int nT1 = t.nT1, nT2 = t.nT2, rows = t.rows, tau2 = t.tau2;
     const int ntiles = nT1 * nT2;
-    const int nitems = ntiles * M;
-    for (int item = threadIdx.x; item < nitems; item += kThreads) {
-        const int mm = item / ntiles;
-        const int tt = item - mm * ntiles;
-        const int tj = tt % nT2, ti = tt / nT2;
-        const int m = mm - l;
-        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);
-        float ar[TI][TJ], ai[TI][TJ];
-        unsigned pa[TI], pb[TJ];
+    const int mm = item / ntiles;
+    const int tt = item - mm * ntiles;
+    const int tj = tt % nT2, ti = tt / nT2;
+    const int m = mm - l;
+    const int lo = max(-l2, m - l1), hi = min(l2, m + l1);
+    it.valid = 0;
 #pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            pa[i] = opaque(lds_addr(f1 + min(ti + nT1 * i, rows - 1) * M1 + (m + l1) - lo));   // walks down
+    for (int i = 0; i < TI; ++i) {
+        it.pa[i] = lds_addr(f1 + min(ti + nT1 * i, rows - 1) * M1 + (m + l1) - lo);
 #pragma unroll
-            for (int j = 0; j < TJ; ++j) ar[i][j] = ai[i][j] = 0.f;
-        }
+        for (int j = 0; j < TJ; ++j)
+            if (ti + nT1 * i < rows && tj + nT2 * j < tau2) it.valid |= 1 << (i * TJ + j);
+    }
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) pb[j] = opaque(lds_addr(f2 + min(tj + nT2 * j, tau2 - 1) * M2 + l2 + lo));
-        unsigned pc = opaque(lds_addr(cg + mm * M2 + l2 + lo));
-        const unsigned pc_end = pc + 4u * (unsigned)(hi - lo);
-        if (hi >= lo) {
+    for (int j = 0; j < TJ; ++j) it.pb[j] = lds_addr(f2 + min(tj + nT2 * j, tau2 - 1) * M2 + l2 + lo);
+    it.pc = lds_addr(cg + mm * M2 + l2 + lo);
+    it.pc_end = it.pc + 4u * (unsigned)(hi - lo);
+    it.any = hi >= lo;
+    it.obase = (ti * tau2 + tj) * M + mm;
+}
+
+// The item's TI x TJ sums for the sample whose fragments lie `bufofs` bytes behind buffer 0.
+template <int TI, int TJ>
+__device__ __forceinline__ void fwd_item_run(const CgTask& t, const FwdItem<TI, TJ>& it, unsigned bufofs,
+                                             float2* __restrict__ out) {
+    float ar[TI][TJ], ai[TI][TJ];
+    unsigned pa[TI], pb[TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        pa[i] = opaque(it.pa[i] + bufofs);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) ar[i][j] = ai[i][j] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) pb[j] = opaque(it.pb[j] + bufofs);
+    unsigned pc = opaque(it.pc);
+    const unsigned pc_end = it.pc_end;
+    if (it.any) {
 #pragma unroll 2
-            for (; pc <= pc_end; pc += 4u) {
-                const float c = lds_f(pc)[0];
-                float2 b[TJ];
+        for (; pc <= pc_end; pc += 4u) {
+            const float c = lds_f(pc)[0];
+            float2 b[TJ];
 #pragma unroll
-                for (int j = 0; j < TJ; ++j) { b[j] = lds_c(pb[j], 0); pb[j] += 8u; }
+            for (int j = 0; j < TJ; ++j) { b[j] = lds_c(pb[j], 0); pb[j] += 8u; }
 #pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    float2 a = lds_c(pa[i], 0);
-                    pa[i] -= 8u;
-                    a.x *= c;
-                    a.y *= c;
+            for (int i = 0; i < TI; ++i) {
+                float2 a = lds_c(pa[i], 0);
+                pa[i] -= 8u;
+                a.x *= c;
+                a.y *= c;
 #pragma unroll
-                    for (int j = 0; j < TJ; ++j) {
-                        ar[i][j] = fmaf(a.x, b[j].x, ar[i][j]);
-                        ar[i][j] = fmaf(-a.y, b[j].y, ar[i][j]);
-                        ai[i][j] = fmaf(a.x, b[j].y, ai[i][j]);
-                        ai[i][j] = fmaf(a.y, b[j].x, ai[i][j]);
-                    }
+                for (int j = 0; j < TJ; ++j) {
+                    ar[i][j] = fmaf(a.x, b[j].x, ar[i][j]);
+                    ar[i][j] = fmaf(-a.y, b[j].y, ar[i][j]);
+                    ai[i][j] = fmaf(a.x, b[j].y, ai[i][j]);
+                    ai[i][j] = fmaf(a.y, b[j].x, ai[i][j]);
                 }
             }
         }
-#pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            const int t1 = ti + nT1 * i;
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) {
-                const int t2 = tj + nT2 * j;
-                if (t1 < rows && t2 < tau2) out[(t1 * tau2 + t2) * M + mm] = make_float2(ar[i][j], ai[i][j]);
-            }
-        }
     }
-}
-
-template <int TI>
-__device__ __forceinline__ void fwd_dispatch_j(const CgTask& t, const float* cg, const float2* f1,
-                                               const float2* f2, float2* out) {
-    switch (t.TJ) {
-        case 1: fwd_tiles<TI, 1>(t, cg, f1, f2, out); break;
-        case 2: fwd_tiles<TI, 2>(t, cg, f1, f2, out); break;
-        case 3: fwd_tiles<TI, 3>(t, cg, f1, f2, out); break;
-        default: fwd_tiles<TI, 4>(t, cg, f1, f2, out); break;
-    }
+    const int M = 2 * t.l + 1;
+    const int si = t.nT1 * t.tau2 * M, sj = t.nT2 * M;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+            if (it.valid & (1 << (i * TJ + j))) out[it.obase + i * si + j * sj] = make_float2(ar[i][j], ai[i][j]);
 }
 
 // LDS of the forward kernel: two fragment buffers (slab of l1 rows, slab of l2) | output tile | table
@@ -222,12 +235,11 @@ __host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
     return ((8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15) + 2 * fwd_frag_lds(t) + 4 * M * M2;
 }
 
-__global__ void __launch_bounds__(kThreads)
-cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const float* __restrict__ CG,
-                  const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
-                  double* __restrict__ stats_part, int sumT) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    const CgTask t = tasks[blockIdx.x];
+template <int TI, int TJ>
+__device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restrict__ F, float2* __restrict__ FF,
+                                          const float* __restrict__ CG, int nF, int nFF, int B,
+                                          int samples_per_group, double* __restrict__ stats_part, int sumT,
+                                          unsigned char* smem) {
     const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
     const int nch = t.rows * t.tau2;
     const int nout = nch * M, n1 = t.rows * M1, n2 = t.tau2 * M2, ncg = M * M2;
@@ -238,6 +250,8 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
     float2* out = reinterpret_cast<float2*>(smem + 2 * frag_bytes);
     float* cg = reinterpret_cast<float*>(smem + 2 * frag_bytes + out_bytes);
     const int tid = threadIdx.x;
+    const float2* f1_0 = reinterpret_cast<const float2*>(frag);
+    const float2* f2_0 = reinterpret_cast<const float2*>(frag + f1_bytes);
 
     // fragments of sample b -> buffer `par`, straight into LDS
     auto issue = [&](int b, int par) {
@@ -250,6 +264,11 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
         if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
     };
 
+    const int nitems = t.nT1 * t.nT2 * M;
+    const bool single = nitems <= kThreads;                       // one item per thread: set up once
+    FwdItem<TI, TJ> mine;
+    if (single && tid < nitems) fwd_item_setup<TI, TJ>(t, tid, cg, f1_0, f2_0, mine);
+
     double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};
     const int b0 = blockIdx.y * samples_per_group;
     const int b1 = min(B, b0 + samples_per_group);
@@ -260,13 +279,15 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
         dma_wait();
         __syncthreads();       // this sample's fragments landed; the previous tile has been copied out
         if (b + 1 < b1) issue(b + 1, par ^ 1);
-        const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
-        const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
-        switch (t.TI) {
-            case 1: fwd_dispatch_j<1>(t, cg, f1, f2, out); break;
-            case 2: fwd_dispatch_j<2>(t, cg, f1, f2, out); break;
-            case 3: fwd_dispatch_j<3>(t, cg, f1, f2, out); break;
-            default: fwd_dispatch_j<4>(t, cg, f1, f2, out); break;
+        const unsigned bufofs = (unsigned)(par * frag_bytes);
+        if (single) {
+            if (tid < nitems) fwd_item_run<TI, TJ>(t, mine, bufofs, out);
+        } else {
+            for (int item = tid; item < nitems; item += kThreads) {
+                FwdItem<TI, TJ> it;
+                fwd_item_setup<TI, TJ>(t, item, cg, f1_0, f2_0, it);
+                fwd_item_run<TI, TJ>(t, it, bufofs, out);
+            }
         }
         __syncthreads();
         // tile -> FF with 16-byte stores from the first 16-byte boundary on
@@ -309,6 +330,24 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
             }
         }
     }
+}
+
+__global__ void __launch_bounds__(kThreads)
+cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const float* __restrict__ CG,
+                  const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
+                  double* __restrict__ stats_part, int sumT) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CgTask t = tasks[blockIdx.x];
+#define CGNET_FWD(TI_, TJ_) \
+    case (TI_) * 8 + (TJ_): fwd_group<TI_, TJ_>(t, F, FF, CG, nF, nFF, B, samples_per_group, stats_part, sumT, smem); break;
+    switch (min(t.TI, 4) * 8 + min(t.TJ, 4)) {
+        CGNET_FWD(1, 1) CGNET_FWD(1, 2) CGNET_FWD(1, 3) CGNET_FWD(1, 4)
+        CGNET_FWD(2, 1) CGNET_FWD(2, 2) CGNET_FWD(2, 3) CGNET_FWD(2, 4)
+        CGNET_FWD(3, 1) CGNET_FWD(3, 2) CGNET_FWD(3, 3) CGNET_FWD(3, 4)
+        CGNET_FWD(4, 1) CGNET_FWD(4, 2) CGNET_FWD(4, 3)
+        default: fwd_group<4, 4>(t, F, FF, CG, nF, nFF, B, samples_per_group, stats_part, sumT, smem); break;
+    }
+#undef CGNET_FWD
 }
 
 __global__ void __launch_bounds__(256)
