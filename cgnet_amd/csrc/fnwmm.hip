@@ -22,7 +22,6 @@
 
 namespace cgnet {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 struct WmmDeg {
     int l, M;          // degree, 2l+1
@@ -187,19 +186,6 @@ pack_w_backward_kernel(const float2* __restrict__ W, const float* __restrict__ s
 }
 
 // --------------------------------------------------------------------------- forward (MFMA)
-__device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-}
-
-// Called between the last matrix instruction of a chain and the first ordinary read of its
-// accumulators: gives the matrix pipeline time to retire its results (an accumulator read
-// hoisted directly behind the chain returned stale values otherwise).
-__device__ __forceinline__ void mfma_drain() {
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
 // Streaming helper: a contiguous run of n complex numbers starting at element `off` of a
 // (16-byte aligned) float2 array is fetched with 16-byte loads, lane-contiguous, from the
 // element pair that contains `off`; the LDS image therefore starts `off & 1` elements early.
