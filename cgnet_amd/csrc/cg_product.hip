@@ -933,15 +933,15 @@ __global__ void __launch_bounds__(256)
 cg_backward_pad_kernel(const float2* __restrict__ F, const float* __restrict__ CG, float2* __restrict__ Fp,
                        float* __restrict__ CGP, const int* __restrict__ meta, int L, int nF, int nFp, int B,
                        int nbF) {
+    __shared__ int s_tab[kMaxLookup];
     const int* cumF = meta;                 // L+2
     const int* cumFp = meta + (L + 2);      // L+2
     const int* tri = cumFp + (L + 2);       // 5 per triple
     if ((int)blockIdx.x < nbF) {
         const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-        if (idx >= (size_t)B * nFp) return;
         const int b = (int)(idx / nFp), e = (int)(idx % nFp);
-        int lam = 0;
-        while (lam < L && cumFp[lam + 1] <= e) ++lam;
+        const int lam = lookup_in_group(L + 1, e, [&](int k) { return cumFp[k]; }, s_tab);
+        if (idx >= (size_t)B * nFp) return;
         const int rel = e - cumFp[lam], Mq = 2 * lam + 2;
         const int t = rel / Mq, x = rel - t * Mq;
         float2 v = make_float2(0.f, 0.f);
@@ -961,15 +961,15 @@ cg_backward_pad_kernel(const float2* __restrict__ F, const float* __restrict__ C
 __global__ void __launch_bounds__(256)
 cg_backward_combine_kernel(const float2* __restrict__ part1, const float2* __restrict__ part2,
                            float2* __restrict__ gF, const int* __restrict__ meta, int L, int nF, int P2, int B) {
+    __shared__ int s_tab[kMaxLookup];
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (size_t)B * nF) return;
     const int b = (int)(idx / nF), e = (int)(idx % nF);
     const int* cumF = meta;                 // L+2
     const int* own1 = meta + (L + 2);       // L+1
     const int* lbeg = own1 + (L + 1);       // L+2
     const int* loff = lbeg + (L + 2);
-    int lam = 0;
-    while (lam < L && cumF[lam + 1] <= e) ++lam;
+    const int lam = lookup_in_group(L + 1, e, [&](int k) { return cumF[k]; }, s_tab);
+    if (idx >= (size_t)B * nF) return;
     const int rel = e - cumF[lam];
     float2 s = make_float2(0.f, 0.f);
     if (own1[lam]) s = part1[idx];

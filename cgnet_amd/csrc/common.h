@@ -53,6 +53,21 @@ private:
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                    \
     } while (0)
 
+// ---- per-thread lookup in a short ascending table -------------------------------------------
+// Index k with base(k) <= x < base(k+1) (k = n-1 if x is past the last base) for a table of n
+// bases that lives in global memory.  The group first copies the table to `s_tab` (n ints of
+// shared memory), so the search itself costs LDS reads instead of a chain of global loads.
+// Every thread of the group must call it (one barrier inside).
+constexpr int kMaxLookup = 64;
+template <typename BaseOf>
+__device__ __forceinline__ int lookup_in_group(int n, int x, BaseOf base_of, int* s_tab) {
+    for (int k = threadIdx.x; k < n; k += blockDim.x) s_tab[k] = base_of(k);
+    __syncthreads();
+    int k = 0;
+    while (k + 1 < n && s_tab[k + 1] <= x) ++k;
+    return k;
+}
+
 // ---- matrix cores -----------------------------------------------------------------------------
 // v_mfma_f32_16x16x4_f32: A[i][k] sits in lane 16*k + i, B[k][j] in lane 16*k + j, and lane n holds
 // D[4*(n/16) + v][n%16] in component v of the accumulator.

@@ -126,10 +126,10 @@ fn_sum_groups_kernel(const double* __restrict__ part, double* __restrict__ sums,
 __global__ void __launch_bounds__(256)
 fn_update_std_kernel(const double* __restrict__ sums, float* __restrict__ stds,
                      const WmmDeg* __restrict__ degs, int ndeg, int sumT, int B, float cnt) {
+    __shared__ int s_tab[kMaxLookup];
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int di = lookup_in_group(ndeg, c, [&](int k) { return degs[k].cumT; }, s_tab);
     if (c >= sumT) return;
-    int di = 0;
-    while (di + 1 < ndeg && degs[di + 1].cumT <= c) ++di;
     const double N = (double)B * (double)degs[di].M;
     const double mean = sums[2 * c] / N;
     double var = sums[2 * c + 1] / N - mean * mean;
@@ -146,11 +146,11 @@ fn_update_std_kernel(const double* __restrict__ sums, float* __restrict__ stds,
 __global__ void __launch_bounds__(256)
 pack_w_forward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                       const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int total_blocks) {
+    __shared__ int s_tab[kMaxLookup];
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     const int blk = idx >> 6;
+    const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].wp_base; }, s_tab);
     if (blk >= total_blocks) return;
-    int di = 0;
-    while (di + 1 < ndeg && degs[di + 1].wp_base <= blk) ++di;
     const WmmDeg d = degs[di];
     // 256 floats per (block of 8 channels, row chunk): lane-major, 4 per lane = (step, re/im rows)
     const int rel = idx - d.wp_base * 64;
@@ -172,10 +172,10 @@ pack_w_forward_kernel(const float2* __restrict__ W, const float* __restrict__ st
 __global__ void __launch_bounds__(256)
 pack_w_backward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                        const WmmDeg* __restrict__ degs, int ndeg, float2* __restrict__ WT, int nW) {
+    __shared__ int s_tab[kMaxLookup];
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int di = lookup_in_group(ndeg, idx, [&](int k) { return degs[k].cumW; }, s_tab);
     if (idx >= nW) return;
-    int di = 0;
-    while (di + 1 < ndeg && degs[di + 1].cumW <= idx) ++di;
     const WmmDeg d = degs[di];
     const int rel = idx - d.cumW;
     const int c = rel / d.tO, to = rel % d.tO;
@@ -404,11 +404,11 @@ template __global__ void wmm_forward_kernel<6>(const float2*, const float*, floa
 __global__ void __launch_bounds__(256)
 wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
                       const int* __restrict__ cumO_S, int ndeg, int B, int nO) {
+    __shared__ int s_tab[kMaxLookup];
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (size_t)B * nO) return;
     const int e = (int)(idx % nO);
-    int di = 0;
-    while (di + 1 < ndeg && cumO_S[di + 1] <= e) ++di;
+    const int di = lookup_in_group(ndeg, e, [&](int k) { return cumO_S[k]; }, s_tab);
+    if (idx >= (size_t)B * nO) return;
     const int S = cumO_S[ndeg + 1 + di];
     float2 s = part[idx];
     for (int k = 1; k < S; ++k) {
@@ -513,7 +513,9 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
 __global__ void __launch_bounds__(256)
 wmm_gradw_finish_kernel(const float2* __restrict__ part, const float* __restrict__ stds, float eps,
                         const WmmDeg* __restrict__ degs, int ndeg, float2* __restrict__ gW, int nW, int nchunks) {
+    __shared__ int s_tab[kMaxLookup];
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int di = lookup_in_group(ndeg, idx, [&](int k) { return degs[k].cumW; }, s_tab);
     if (idx >= nW) return;
     float2 s = part[idx];
     for (int k = 1; k < nchunks; ++k) {
@@ -522,8 +524,6 @@ wmm_gradw_finish_kernel(const float2* __restrict__ part, const float* __restrict
         s.y += v.y;
     }
     if (stds) {
-        int di = 0;
-        while (di + 1 < ndeg && degs[di + 1].cumW <= idx) ++di;
         const WmmDeg d = degs[di];
         const int c = (idx - d.cumW) % d.K;
         const float r = fmaxf(eps, stds[d.cumT + c]);
@@ -574,11 +574,11 @@ wmm_gradff_kernel(const float2* __restrict__ gO, const float2* __restrict__ WT, 
 __global__ void __launch_bounds__(256)
 pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                      const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Ap, int total_blocks) {
+    __shared__ int s_tab[kMaxLookup];
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     const int blk = idx >> 6, lane = idx & 63;
+    const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].ap_base; }, s_tab);
     if (blk >= total_blocks) return;
-    int di = 0;
-    while (di + 1 < ndeg && degs[di + 1].ap_base <= blk) ++di;
     const WmmDeg d = degs[di];
     const int rel = blk - d.ap_base;             // ctile * nks_b + ks
     const int ks = rel % d.nks_b, ctile = rel / d.nks_b;
