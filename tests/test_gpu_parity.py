@@ -89,15 +89,15 @@ def test_cg_table_matches_oracle(dev, lmax, mode):
 # ------------------------------------------------------------------------------- CG product
 CG_CASES = [
     # lmax, taus, B, mode
-    (3, [2, 2, 2, 2], 4, "default"),                      # BASELINE config 1
+    (3, [2, 2, 2, 2], 4, "default"),                      # benchmark configuration 1
     (3, [2, 2, 2, 2], 4, "mst"),
     (4, [3, 1, 0, 5, 2], 3, "default"),                   # ragged, a degree without channels
     (2, [1, 1, 1], 1, "default"),                         # tau = 1 everywhere, single sample
     (5, [7, 6, 5, 13, 3, 9], 5, "mst"),
     (6, [17, 4, 4, 4, 4, 4, 33], 2, "debug"),             # more than 16 channels in the reduced slot
-    (11, [5] * 12, 6, "default"),                         # BASELINE config 2 shape, small batch
-    (11, [12] * 12, 3, "default"),                        # BASELINE config 3 shape, small batch
-    (15, [16] * 16, 2, "mst"),                            # BASELINE config 4 shape, small batch
+    (11, [5] * 12, 6, "default"),                         # benchmark configuration 2 shape, small batch
+    (11, [12] * 12, 3, "default"),                        # benchmark configuration 3 shape, small batch
+    (15, [16] * 16, 2, "mst"),                            # benchmark configuration 4 shape, small batch
 ]
 
 
@@ -277,8 +277,8 @@ LAYER_CASES = [
     (3, [2, 2, 2, 2], [2, 2, 2, 2], 4, False, True),
     (3, [2, 2, 2, 2], [3, 1, 2, 2], 4, True, True),
     (4, [3, 2, 1, 2, 2], [2, 2, 2, 2, 2], 3, False, False),
-    (11, [5] * 12, [5] * 12, 8, False, True),            # BASELINE config 2 shape (B reduced for the oracle)
-    (11, [12] * 12, [12] * 12, 3, False, True),          # BASELINE config 3 shape (B reduced)
+    (11, [5] * 12, [5] * 12, 8, False, True),            # benchmark configuration 2 shape (B reduced for the oracle)
+    (11, [12] * 12, [12] * 12, 3, False, True),          # benchmark configuration 3 shape (B reduced)
 ]
 
 
@@ -394,7 +394,7 @@ def test_spherical_cnn_stack(dev):
 
 # ------------------------------------------------------------------------------- full-size properties
 def test_full_size_properties_config3(dev):
-    """BASELINE config 3 (L=11, tau=12, B=100): properties that need no CPU-sized oracle."""
+    """benchmark configuration 3 (L=11, tau=12, B=100): properties that need no CPU-sized oracle."""
     from cgnet_amd import CG_layers
     lmax, taus, bsz = 11, [12] * 12, 100
     mod = CG_layers.CG_woFilter_cuda(lmax, taus, device=dev)
@@ -459,7 +459,7 @@ def test_full_size_layer_config3_runs(dev):
 
 @pytest.mark.parametrize("sparse", [True, False])
 def test_full_size_properties_config4(dev, sparse):
-    """BASELINE config 4 (L=15, tau=16, B=64, MST and default triples): CG product forward + backward."""
+    """benchmark configuration 4 (L=15, tau=16, B=64, MST and default triples): CG product forward + backward."""
     from cgnet_amd import CG_layers
     lmax, taus, bsz = 15, [16] * 16, 64
     mod = CG_layers.CG_woFilter_cuda(lmax, taus, lll_mode="mst" if sparse else None, device=dev)
@@ -485,7 +485,7 @@ def test_full_size_properties_config4(dev, sparse):
 
 
 def test_full_size_stack_config5_runs(dev):
-    """BASELINE config 5 (L=20, taus 1 -> 16 x 4, B=32): SphericalCNN embedding, linear head, cross-entropy."""
+    """benchmark configuration 5 (L=20, taus 1 -> 16 x 4, B=32): SphericalCNN embedding, linear head, cross-entropy."""
     from cgnet_amd import CGNet
     lmax, bsz = 20, 32
     taus = [[1] * 21] + [[16] * 21] * 4
