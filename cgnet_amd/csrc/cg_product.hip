@@ -137,7 +137,7 @@ __device__ __forceinline__ float sqrt_refined(float n) {
 }
 
 // One item = one m of a TI x TJ tile of channels.  Items are ordered m-major, so the lanes of a
-// wave work on neighbouring m (similar numbers of terms) of all channel tiles.  What an item needs
+// wave work on a few m with similar numbers of terms, for all channel tiles.  What an item needs
 // to know does not depend on the sample: it is worked out once per group.
 template <int TI, int TJ>
 struct FwdItem {
@@ -155,8 +155,11 @@ __device__ __forceinline__ void fwd_item_setup(const CgTask& t, int item, const 
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int nT1 = t.nT1, nT2 = t.nT2, rows = t.rows, tau2 = t.tau2;
     const int ntiles = nT1 * nT2;
-    const int mm = item / ntiles;
-    const int tt = item - mm * ntiles;
+    // m numbered from the middle of the axis outwards: the waves with the many-term middle m are
+    // full, the last (partly filled) wave gets the outer m with few terms
+    const int mslot = item / ntiles;
+    const int tt = item - mslot * ntiles;
+    const int mm = (mslot & 1) ? l + ((mslot + 1) >> 1) : l - (mslot >> 1);
     const int tj = tt % nT2, ti = tt / nT2;
     const int m = mm - l;
     const int lo = max(-l2, m - l1), hi = min(l2, m + l1);
