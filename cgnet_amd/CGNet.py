@@ -53,6 +53,21 @@ class SphericalCNN(nn.Module):
         return fs[0].reshape(B, -1)
 
 
+def normalisation_counts(module):
+    """{module path: bn_cnt} of every fragment-normalisation layer under ``module``.  The count is a plain
+    python attribute in the reference (``CG_layers.py:92,130``) and therefore missing from ``state_dict``;
+    store this dict next to a checkpoint and hand it to ``load_normalisation_counts`` when resuming."""
+    return {name: float(m.bn_cnt) for name, m in module.named_modules() if hasattr(m, "bn_cnt")}
+
+
+def load_normalisation_counts(module, counts):
+    named = dict(module.named_modules())
+    for name, cnt in counts.items():
+        if name not in named or not hasattr(named[name], "bn_cnt"):
+            raise KeyError("no fragment-normalisation layer named %r" % name)
+        named[name].bn_cnt = float(cnt)
+
+
 # The reference's README and Shrec17 script name a "SphericalCNN_fast"; its source is not part
 # of the reference, so only the name can be honoured.
 SphericalCNN_fast = SphericalCNN

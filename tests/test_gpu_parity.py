@@ -522,6 +522,54 @@ def test_full_size_stack_config5_runs(dev):
     assert got == pytest.approx(want, rel=5e-2, abs=1e-5)
 
 
+def test_classifier_from_coefficient_file(dev, tmp_path):
+    """Coefficient file -> straight batch -> MNIST_Net: the first layer against the oracle, the head end to end."""
+    from cgnet_amd import CGNet, data, model
+    n_deg, bsz = 4, 6
+    rng = np.random.default_rng(3)
+    coefs = rng.standard_normal((10, 25)) + 1j * rng.standard_normal((10, 25))     # computed for 5 degrees
+    np.save(tmp_path / "L_5.npy", coefs)
+    np.save(tmp_path / "label.npy", np.arange(10))
+    ds = data.CoefficientFile(str(tmp_path / "L_5.npy"), n_deg, str(tmp_path / "label.npy"))
+    x = ds.batch(range(bsz)).to(dev)
+    assert tuple(x.shape) == (bsz, n_deg * n_deg, 2)
+    net = model.MNIST_Net(n_deg - 1, tau_type=2, tau_man=4, nlayers=2, dropout=None)
+    # layer 0 alone against the oracle (injected weights and statistics)
+    cg0 = net.SphericalCNN.cgs[0]
+    taus_in, taus_out = [1] * n_deg, model.define_taus(2, 4, n_deg - 1)
+    ora = OL.LayerOracle(n_deg - 1, taus_in, taus_out, cg0.cg.lll_list, batchnorm=True)
+    g = torch.Generator().manual_seed(0)
+    t_ff = [int(v) for v in cg0.t_FF]
+    w64 = torch.randn(sum(a * b for a, b in zip(t_ff, taus_out)), 2, generator=g, dtype=torch.float64) * 0.3
+    stds = 0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
+    with torch.no_grad():
+        cg0.bnWMM.W.copy_(w64.float())
+        cg0.bnWMM.bn_stds.copy_(stds.float())
+    ora.set_stds_flat(stds.float().double().numpy())
+    ora.training = False
+    cg0.eval()
+    want = OL.join_straight(ora.forward(x.double().cpu(), w64.float().double()))
+    assert_close(cg0(x, straight_output=True), want, "first layer on file input")
+    # the whole classifier
+    net.train()
+    logp = net(x)
+    assert tuple(logp.shape) == (bsz, 10)
+    assert torch.allclose(logp.exp().sum(1), torch.ones(bsz, device=dev), atol=1e-5)
+    labels = torch.tensor([ds[i][1] for i in range(bsz)], device=dev)
+    torch.nn.functional.nll_loss(logp, labels).backward()
+    for p in net.parameters():
+        if p.requires_grad:
+            assert p.grad is not None and torch.isfinite(p.grad).all()
+    counts = CGNet.normalisation_counts(net)
+    assert counts == {"SphericalCNN.cgs.0.bnWMM": 2.0, "SphericalCNN.cgs.1.bnWMM": 2.0}
+    net2 = model.MNIST_Net(n_deg - 1, tau_type=2, tau_man=4, nlayers=2, dropout=None)
+    net2.load_state_dict(net.state_dict())
+    CGNet.load_normalisation_counts(net2, counts)
+    assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
+    net.eval(); net2.eval()
+    assert torch.equal(net(x), net2(x))
+
+
 # ------------------------------------------------------------------------------- error behaviour
 def test_errors(dev):
     from cgnet_amd import CG_cuda_ops, CG_layers, _plans
