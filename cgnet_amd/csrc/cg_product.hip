@@ -309,15 +309,17 @@ __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restr
             for (int k = 0; k < 4; ++k) {
                 const int ch = tid + kThreads * k;
                 if (ch < nch) {
-                    float a = 0.f, q = 0.f;
+                    // both sums run over the same rounded |z| in double: the variance formed from them
+                    // later is then free of cancellation between inconsistently rounded terms
+                    double a = s1[k], q = s2[k];
                     for (int mm = 0; mm < M; ++mm) {
                         const float2 z = out[ch * M + mm];
-                        const float n = fmaf(z.x, z.x, z.y * z.y);
-                        q += n;
-                        a += sqrt_refined(n);
+                        const double r = (double)sqrt_refined(fmaf(z.x, z.x, z.y * z.y));
+                        a += r;
+                        q = fma(r, r, q);
                     }
-                    s1[k] += (double)a;
-                    s2[k] += (double)q;
+                    s1[k] = a;
+                    s2[k] = q;
                 }
             }
         }

@@ -94,15 +94,14 @@ fn_stats_kernel(const float2* __restrict__ FF, const WmmDeg* __restrict__ degs,
         for (int e = tid; e < n; e += kThreads) tile[e] = src[e];
         __syncthreads();
         if (tid < u.nc) {
-            float a = 0.f, q = 0.f;
+            // both sums run over the same rounded |z| in double (no cancellation between
+            // inconsistently rounded terms when the variance is formed)
             for (int mm = 0; mm < d.M; ++mm) {
                 const float2 z = tile[tid * d.M + mm];
-                const float nn = fmaf(z.x, z.x, z.y * z.y);
-                q += nn;
-                a += sqrtf(nn);
+                const double r = (double)sqrtf(fmaf(z.x, z.x, z.y * z.y));
+                s1 += r;
+                s2 = fma(r, r, s2);
             }
-            s1 += (double)a;
-            s2 += (double)q;
         }
         __syncthreads();
     }

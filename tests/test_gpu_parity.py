@@ -343,6 +343,41 @@ def test_layer_forward_backward(dev, lmax, tin, tout, bsz, sparse, bn, fused):
             assert_close(a, b, "eval forward")
 
 
+def _random_layer_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for k in range(n):
+        lmax = int(rng.integers(1, 9))
+        hi = int(rng.choice([3, 9, 18]))
+        tin = [int(rng.integers(0 if l > 0 else 1, hi + 1)) for l in range(lmax + 1)]
+        tout = [int(rng.integers(1, hi + 1)) for _ in range(lmax + 1)]
+        bsz = int(rng.integers(1, 12))
+        cases.append((lmax, tin, tout, bsz, bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0), k))
+    return cases
+
+
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _random_layer_cases(24, 2024))
+def test_layer_random_shapes(dev, lmax, tin, tout, bsz, sparse, bn, k):
+    """Seeded random degrees, ragged channel counts (zero channels included), batch sizes and triple sets:
+    one training step of the layer, forward and both gradients, against the oracle."""
+    mod, ora, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=100 + k)
+    x64 = rand_straight(tin, bsz, seed=200 + k)
+    g = torch.Generator().manual_seed(300 + k)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
+    xo = x64.float().double().requires_grad_(True)
+    wo = w64.clone().requires_grad_(True)
+    want = OL.join_straight(ora.forward(xo, wo))
+    want_gx, want_gw = torch.autograd.grad(want, (xo, wo), go64, allow_unused=True)
+    x = x64.float().to(dev).requires_grad_(True)
+    out = mod(x, straight_output=True)
+    assert_close(out, want, "layer forward")
+    out.backward(go64.float().to(dev))
+    assert_close(x.grad, want_gx if want_gx is not None else torch.zeros_like(xo), "layer grad F")
+    if wo.numel():
+        assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W")
+
+
 def test_spherical_cnn_stack(dev):
     from cgnet_amd import CGNet
     lmax = 4
