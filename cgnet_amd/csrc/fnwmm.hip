@@ -55,13 +55,14 @@ struct cgnet_wmm_plan {
     std::vector<cgnet::WmmDeg> degs;
     std::vector<cgnet::WmmFwdUnit> fwd_units;   // units of degrees with NC <= 3 first
     int fwd_units_small = 0;
-    std::vector<cgnet::WmmChanUnit> gw_units, gw_units_rc0, gff_units, stat_units;
+    std::vector<cgnet::WmmChanUnit> gw_units, gw_units_rc0, gff_units, gff_zero_units, stat_units;
     std::vector<int> cumO_all, cumFF_all;   // L+2 entries, for element -> degree lookups
     cgnet::WmmDeg* d_degs = nullptr;
     cgnet::WmmFwdUnit* d_fwd_units = nullptr;
     cgnet::WmmChanUnit* d_gw_units = nullptr;
     cgnet::WmmChanUnit* d_gw_units_rc0 = nullptr;   // one entry per 64-channel chunk (row chunk 0 only)
     cgnet::WmmChanUnit* d_gff_units = nullptr;
+    cgnet::WmmChanUnit* d_gff_zero_units = nullptr;   // channels of degrees without outputs: their gradient is zero
     cgnet::WmmChanUnit* d_stat_units = nullptr;
     int* d_cumO = nullptr;      // per deg index: cumO, and S, interleaved: [ndeg+1] cumO then [ndeg] S
     size_t stat_lds = 0, gff_lds = 0;
@@ -756,7 +757,7 @@ using namespace cgnet;
 
 static void free_plan(cgnet_wmm_plan* plan) {
     if (!plan) return;
-    void* ptrs[] = {plan->d_degs, plan->d_fwd_units, plan->d_gw_units, plan->d_gw_units_rc0, plan->d_gff_units,
+    void* ptrs[] = {plan->d_degs, plan->d_fwd_units, plan->d_gw_units, plan->d_gw_units_rc0, plan->d_gff_units, plan->d_gff_zero_units,
                     plan->d_stat_units, plan->d_cumO};
     for (void* q : ptrs)
         if (q) (void)hipFree(q);
@@ -845,8 +846,10 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
             p->stat_units.push_back(WmmChanUnit{di, 0, c0, std::min(per_stat, d.K - c0)});
         p->stat_lds = std::max(p->stat_lds, (size_t)8 * per_stat * d.M);
         const int per_gff = std::max(1, 4096 / d.M);
-        for (int c0 = 0; c0 < d.K; c0 += per_gff)
+        for (int c0 = 0; c0 < d.K; c0 += per_gff) {
             p->gff_units.push_back(WmmChanUnit{di, 0, c0, std::min(per_gff, d.K - c0)});
+            if (d.tO == 0) p->gff_zero_units.push_back(p->gff_units.back());
+        }
         p->gff_lds = std::max(p->gff_lds, (size_t)8 * d.tO * d.M);
     }
     // the matrix-core gradient kernel keeps a tile and two operand buffers per wave inside 64 KB of LDS
@@ -891,6 +894,7 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         if (u.rc == 0) p->gw_units_rc0.push_back(u);
     if ((rc = upload(p->gw_units_rc0.data(), sizeof(WmmChanUnit) * p->gw_units_rc0.size(), (void**)&p->d_gw_units_rc0))) return rc;
     if ((rc = upload(p->gff_units.data(), sizeof(WmmChanUnit) * p->gff_units.size(), (void**)&p->d_gff_units))) return rc;
+    if ((rc = upload(p->gff_zero_units.data(), sizeof(WmmChanUnit) * p->gff_zero_units.size(), (void**)&p->d_gff_zero_units))) return rc;
     if ((rc = upload(p->stat_units.data(), sizeof(WmmChanUnit) * p->stat_units.size(), (void**)&p->d_stat_units))) return rc;
     if ((rc = upload(cumO_S.data(), sizeof(int) * cumO_S.size(), (void**)&p->d_cumO))) return rc;
     *plan = guard.release();
@@ -1075,6 +1079,13 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
                          dim3(kThreads), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
                          plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, out_bytes, go_bytes);
             CGNET_HIP(hipGetLastError());
+            if (!plan->gff_zero_units.empty()) {
+                // degrees that produce no output channels: the general kernel writes their zeros
+                CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_zero_units.size(), B), dim3(kThreads),
+                             plan->gff_lds, s, (const float2*)d_gO, (const float2*)nullptr, (float2*)d_gFF,
+                             plan->d_degs, plan->d_gff_zero_units, plan->nFF, plan->nO);
+                CGNET_HIP(hipGetLastError());
+            }
         } else {
             if (plan->nW > 0) {
                 CGNET_LAUNCH(pack_w_backward_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,

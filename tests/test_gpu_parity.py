@@ -135,6 +135,25 @@ def test_cg_forward_backward(dev, lmax, taus, bsz, mode):
     assert torch.equal(torch.cat([p.reshape(bsz, -1, 2) for p in y_list], 1), y.detach())
 
 
+def _random_cg_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        lmax = int(rng.integers(0, 10))
+        hi = int(rng.choice([2, 7, 20, 36]))
+        if lmax > 6:
+            hi = min(hi, 7)                                # keeps the CPU oracle in seconds
+        taus = [int(rng.integers(0 if l > 0 else 1, hi + 1)) for l in range(lmax + 1)]
+        cases.append((lmax, taus, int(rng.integers(1, 9)), str(rng.choice(["default", "mst", "debug"]))))
+    return cases
+
+
+@pytest.mark.parametrize("lmax,taus,bsz,mode", _random_cg_cases(24, 11))
+def test_cg_random_shapes(dev, lmax, taus, bsz, mode):
+    """Seeded random degrees, ragged channel counts (beyond 16 and 32 included), batches and triple sets."""
+    test_cg_forward_backward(dev, lmax, taus, bsz, mode)
+
+
 @pytest.mark.parametrize("lmax,taus,bsz,mode", [CG_CASES[2], CG_CASES[5], CG_CASES[7]])
 def test_cg_backward_general_kernel(dev, monkeypatch, lmax, taus, bsz, mode):
     """The LDS-accumulator backward kernel (fallback for shapes the register-resident scheme cannot
@@ -221,8 +240,31 @@ WMM_CASES = [
 ]
 
 
+def _random_wmm_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        lmax = int(rng.integers(0, 13))
+        kmax = int(rng.choice([6, 40, 300]))
+        omax = int(rng.choice([3, 12, 20]))
+        t_ff = [int(rng.integers(0, kmax + 1)) if rng.random() > 0.1 else 0 for _ in range(lmax + 1)]
+        t_out = [int(rng.integers(0, omax + 1)) if rng.random() > 0.1 else 0 for _ in range(lmax + 1)]
+        cases.append((lmax, t_ff, t_out, int(rng.integers(1, 40)), bool(rng.integers(0, 4) > 0), bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("lmax,t_ff,t_out,bsz,bn,training", _random_wmm_cases(24, 7))
+def test_fn_wmm_random_shapes(dev, lmax, t_ff, t_out, bsz, bn, training):
+    """Seeded random degrees, channel counts (zeros, t_O above 16, counts that are no multiple of 8) and batches."""
+    check_fn_wmm(dev, lmax, t_ff, t_out, bsz, bn, training)
+
+
 @pytest.mark.parametrize("lmax,t_ff,t_out,bsz,bn,training", WMM_CASES)
 def test_fn_wmm_forward_backward(dev, lmax, t_ff, t_out, bsz, bn, training):
+    check_fn_wmm(dev, lmax, t_ff, t_out, bsz, bn, training)
+
+
+def check_fn_wmm(dev, lmax, t_ff, t_out, bsz, bn, training):
     from cgnet_amd import CG_layers
     g = torch.Generator().manual_seed(1000 + lmax + bsz)
     ff64 = rand_straight(t_ff, bsz, seed=5) * 0.3
