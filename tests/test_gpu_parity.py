@@ -385,23 +385,24 @@ def test_layer_forward_backward(dev, lmax, tin, tout, bsz, sparse, bn, fused):
             assert_close(a, b, "eval forward")
 
 
-def _random_layer_cases(n, seed):
+def _random_layer_cases(n, seed, out_lo=1):
     rng = np.random.default_rng(seed)
     cases = []
     for k in range(n):
         lmax = int(rng.integers(1, 9))
         hi = int(rng.choice([3, 9, 18]))
         tin = [int(rng.integers(0 if l > 0 else 1, hi + 1)) for l in range(lmax + 1)]
-        tout = [int(rng.integers(1, hi + 1)) for _ in range(lmax + 1)]
+        tout = [int(rng.integers(out_lo, hi + 1)) for _ in range(lmax + 1)]
         bsz = int(rng.integers(1, 12))
         cases.append((lmax, tin, tout, bsz, bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0), k))
     return cases
 
 
-@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _random_layer_cases(24, 2024))
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k",
+                         _random_layer_cases(24, 2024) + _random_layer_cases(12, 77, out_lo=0))
 def test_layer_random_shapes(dev, lmax, tin, tout, bsz, sparse, bn, k):
-    """Seeded random degrees, ragged channel counts (zero channels included), batch sizes and triple sets:
-    one training step of the layer, forward and both gradients, against the oracle."""
+    """Seeded random degrees, ragged channel counts (degrees without input or without output channels
+    included), batch sizes and triple sets: one training step of the layer, forward and both gradients, against the oracle."""
     mod, ora, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=100 + k)
     x64 = rand_straight(tin, bsz, seed=200 + k)
     g = torch.Generator().manual_seed(300 + k)
