@@ -300,7 +300,7 @@ __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restr
         float4* dst4 = reinterpret_cast<float4*>(dst + head);
         for (int e = tid; e < npair; e += kThreads) {
             const float2 u = out[head + 2 * e], v = out[head + 2 * e + 1];
-            dst4[e] = make_float4(u.x, u.y, v.x, v.y);
+            stream_store16(dst4 + e, u.x, u.y, v.x, v.y);
         }
         if (tid == 0 && head) dst[0] = out[0];
         if (tid == 1 && ((nout - head) & 1)) dst[nout - 1] = out[nout - 1];

@@ -109,6 +109,16 @@ __device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, in
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
 }
 
+// 16-byte store of data that is not read again soon: marked non-temporal, so a long output stream
+// does not push the (small, re-read) operands of the kernel out of the L2 cache.
+__device__ __forceinline__ void stream_store16(void* dst, float a, float b, float c, float d) {
+#ifdef CGNET_NO_STREAM_HINT
+    *reinterpret_cast<f32x4*>(dst) = (f32x4){a, b, c, d};
+#else
+    __builtin_nontemporal_store((f32x4){a, b, c, d}, reinterpret_cast<f32x4*>(dst));
+#endif
+}
+
 // All copies (and loads) this wave has started have landed (vmcnt == 0).
 __device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 

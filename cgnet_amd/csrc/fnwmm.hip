@@ -595,32 +595,36 @@ pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ std
 }
 
 // Gradient with respect to FF on the matrix cores (t_O <= 16): gFF[c, (m, re/im)] = sum_k A[c, k] * B[k, (m, re/im)]
-// with k = (to, re/im).  Every wave works alone (no barrier): it owns 16 channels of the unit and
-// walks over the samples of its group.  The gO rows of the next sample arrive by LDS-direct loads
-// while the current one is multiplied; the 16 x 2M result tile goes through the wave's LDS image
-// and leaves as one contiguous run of 16-byte stores, one sample behind the arithmetic, so the
-// wait for the next operands never waits for fresh stores.
-// NT = column tiles worked on together (all of them when the degree has at most three)
-template <int NKS, int NT>
+// with k = (to, re/im).  A work-group is one wave (no barrier): it owns the up to 64 channels of its
+// unit as tiles of 16, keeps their A operands in registers and walks over the samples of its group.
+// The gO rows of the next sample arrive by LDS-direct loads while the current one is multiplied;
+// one load of the rows serves all channel tiles.  Every 16 x 2M result tile goes through the wave's
+// LDS image and leaves as one contiguous run of 16-byte stores, one tile behind the arithmetic.
+// NT = column tiles worked on together; ONE: these are all column tiles of the degree, so the B
+// operands are built once per sample and shared by the channel tiles.
+constexpr int kGffSub = 4;     // channel tiles per wave
+template <int NKS, int NT, bool ONE>
 __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, const float* __restrict__ Ap,
                                                 float2* __restrict__ gFF, const WmmDeg& d, const WmmChanUnit& u, int B,
                                                 int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes,
-                                                unsigned char* mine, int w, int lane) {
+                                                unsigned char* mine, int lane) {
     float* ol = reinterpret_cast<float*>(mine);                              // [16][2M]
     unsigned char* gobuf = mine + out_bytes;                                  // [2][go_bytes]
     const int i = lane & 15, kk = lane >> 4;
     const int M = d.M, tO = d.tO;
     constexpr int nks = NKS;
-    const int ctile = (u.c0 >> 4) + w;
-    float a[NKS];
+    const int nsub = (u.nc + 15) >> 4;
+    float a[kGffSub][NKS];
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) a[ks] = Ap[((size_t)d.ap_base + (size_t)ctile * nks + ks) * 64 + lane];
+    for (int sub = 0; sub < kGffSub; ++sub)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+            a[sub][ks] = sub < nsub ? Ap[((size_t)d.ap_base + (size_t)((u.c0 >> 4) + sub) * nks + ks) * 64 + lane] : 0.f;
     // k = 4*ks + kk  ->  to = 2*ks + (kk >> 1), re/im = kk & 1;  column 16*ct + i -> m = 8*ct + (i >> 1), re/im = i & 1
     const int to_lane = kk >> 1, sel = kk & 1, r = i & 1;
     const float cx = (r == sel) ? (r ? -1.f : 1.f) : 0.f, cy = (r == sel) ? 0.f : 1.f;   // B = cx * re + cy * im
     const int nct = (2 * M + 15) >> 4;
-    const int rows = min(16, u.nc - 16 * w);
-    const int n_go = tO * M, n_out = rows * M;    // complex entries of the gO rows / of this wave's output run
+    const int n_go = tO * M;                      // complex entries of the gO rows
     const int b_begin = blockIdx.y * samples_per_group, b_end = min(B, b_begin + samples_per_group);
     if (b_begin >= b_end) return;
     {
@@ -634,8 +638,10 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
         dma16<64>(src, dst, n_go >> 1, lane);
         if (n_go & 1) dma8(src + (n_go - 1), dst + 8 * (size_t)(n_go - 1), lane);
     };
-    auto store_tile = [&](int b) {
-        const size_t off = (size_t)b * nFF + d.cumFF + (size_t)(u.c0 + 16 * w) * M;
+    auto rows_of = [&](int sub) { return min(16, u.nc - 16 * sub); };
+    auto store_tile = [&](int b, int sub) {
+        const size_t off = (size_t)b * nFF + d.cumFF + (size_t)(u.c0 + 16 * sub) * M;
+        const int n_out = rows_of(sub) * M;
         float2* dst = gFF + off;
         const float2* src = reinterpret_cast<const float2*>(ol);
         const int head = (int)(off & 1);          // unaligned first entry
@@ -643,81 +649,99 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
         const int n4 = (n_out - head) >> 1;
         for (int idx = lane; idx < n4; idx += 64) {
             const float2 z0 = src[head + 2 * idx], z1 = src[head + 2 * idx + 1];
-            *reinterpret_cast<float4*>(dst + head + 2 * idx) = make_float4(z0.x, z0.y, z1.x, z1.y);
+            stream_store16(dst + head + 2 * idx, z0.x, z0.y, z1.x, z1.y);
         }
         if (((n_out - head) & 1) && lane == 0) dst[n_out - 1] = src[n_out - 1];
     };
+    // lower bound of the store instructions of one tile (the loop of store_tile, without head and tail)
+    auto stores_of = [&](int sub) { return (((rows_of(sub) * M - 1) >> 1) + 63) >> 6; };
+    // Vector memory operations complete in the order issued.  The copy of sample b is started at the
+    // beginning of sample b-1 and followed there by the stores of the last tile of sample b-2 and of
+    // all tiles but the last of sample b-1: waiting until no more than that many operations are
+    // outstanding is enough for the copy and leaves those stores in flight.
+    int later_stores = 0;
+    for (int sub = 0; sub + 1 < nsub; ++sub) later_stores += stores_of(sub);
+    const int last_stores = stores_of(nsub - 1);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the clearing stores precede the first copy
     issue(b_begin, 0);
-    const int row0 = 4 * kk;                      // D rows of this lane inside the wave's tile
+    const int row0 = 4 * kk;                      // D rows of this lane inside a tile
     int par = 0;
     for (int b = b_begin; b < b_end; ++b, par ^= 1) {
-        dma_wait();                               // gO rows of sample b are in LDS
-        asm volatile("" ::: "memory");
-        if (b > b_begin) store_tile(b - 1);
+        wait_vmcnt(b == b_begin ? 0 : later_stores + (b - 2 >= b_begin ? last_stores : 0));   // gO rows of sample b landed
         if (b + 1 < b_end) issue(b + 1, par ^ 1);
         const float2* g = reinterpret_cast<const float2*>(gobuf + (size_t)par * go_bytes);
-        for (int ct0 = 0; ct0 < nct; ct0 += NT) {
-            f32x4 acc[NT];
+        float bv[NKS][NT];
+        auto build_b = [&](int ct0) {
             int mofs[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                mofs[t] = min(8 * (ct0 + t) + (i >> 1), M - 1);           // clamped: extra columns are not stored
-            }
-            float bv[NKS][NT];
+            for (int t = 0; t < NT; ++t) mofs[t] = min(8 * (ct0 + t) + (i >> 1), M - 1);   // clamped: extra columns are not stored
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
-                const int to = min(2 * ks + to_lane, tO - 1);             // clamped: rows past t_O carry zero weights
+                const int to = min(2 * ks + to_lane, tO - 1);                 // clamped: rows past t_O carry zero weights
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     const float2 z = g[to * M + mofs[t]];
                     bv[ks][t] = fmaf(z.x, cx, z.y * cy);
                 }
             }
+        };
+        if (ONE) build_b(0);
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks)
+        for (int sub = 0; sub < kGffSub; ++sub) {
+            if (sub < nsub) {
+                // the tile before this one leaves (its LDS image is read before it is overwritten below)
+                if (sub > 0) store_tile(b, sub - 1);
+                else if (b > b_begin) store_tile(b - 1, nsub - 1);
+                for (int ct0 = 0; ct0 < nct; ct0 += NT) {
+                    if (!ONE) build_b(ct0);
+                    f32x4 acc[NT];
 #pragma unroll
-                for (int t = 0; t < NT; ++t) acc[t] = mfma4(a[ks], bv[ks][t], acc[t]);
-            mfma_drain();
+                    for (int t = 0; t < NT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const int col = (ct0 + t) * 16 + i;
-                if (col < 2 * M) {
+                    for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) ol[(size_t)(row0 + v) * 2 * M + col] = acc[t][v];
+                        for (int t = 0; t < NT; ++t) acc[t] = mfma4(a[sub][ks], bv[ks][t], acc[t]);
+                    mfma_drain();
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const int col = (ct0 + t) * 16 + i;
+                        if (col < 2 * M) {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) ol[(size_t)(row0 + v) * 2 * M + col] = acc[t][v];
+                        }
+                    }
+                    if (ONE) break;
                 }
             }
         }
     }
-    store_tile(b_end - 1);
+    store_tile(b_end - 1, nsub - 1);
 }
 
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(64)
 wmm_gradff_mfma_kernel(const float2* __restrict__ gO, const float* __restrict__ Ap, float2* __restrict__ gFF,
                        const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
                        int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes) {
     extern __shared__ __align__(16) unsigned char smem[];
     const WmmChanUnit u = units[blockIdx.x];
     const WmmDeg d = degs[u.deg];
-    const int lane = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (16 * w >= u.nc) return;                   // wave-uniform; the kernel has no barrier
-    unsigned char* mine = smem + (size_t)w * (out_bytes + 2 * go_bytes);
-#define CGNET_GFF_ARGS gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, mine, w, lane
+    const int lane = threadIdx.x;
+#define CGNET_GFF_ARGS gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, smem, lane
 #define CGNET_GFF(N_)                                                                     \
     case N_:                                                                              \
-        if (nct == 1) wmm_gradff_wave<N_, 1>(CGNET_GFF_ARGS);                             \
-        else if (nct == 2) wmm_gradff_wave<N_, 2>(CGNET_GFF_ARGS);                        \
-        else wmm_gradff_wave<N_, 3>(CGNET_GFF_ARGS);                                      \
+        if (nct == 1) wmm_gradff_wave<N_, 1, true>(CGNET_GFF_ARGS);                       \
+        else if (nct == 2) wmm_gradff_wave<N_, 2, true>(CGNET_GFF_ARGS);                  \
+        else if (nct == 3) wmm_gradff_wave<N_, 3, true>(CGNET_GFF_ARGS);                  \
+        else wmm_gradff_wave<N_, 3, false>(CGNET_GFF_ARGS);                               \
         break;
     const int nct = (2 * d.M + 15) >> 4;
     switch (d.nks_b) {
         CGNET_GFF(1) CGNET_GFF(2) CGNET_GFF(3) CGNET_GFF(4) CGNET_GFF(5) CGNET_GFF(6) CGNET_GFF(7)
         default:
-            if (nct == 1) wmm_gradff_wave<8, 1>(CGNET_GFF_ARGS);
-            else if (nct == 2) wmm_gradff_wave<8, 2>(CGNET_GFF_ARGS);
-            else wmm_gradff_wave<8, 3>(CGNET_GFF_ARGS);
+            if (nct == 1) wmm_gradff_wave<8, 1, true>(CGNET_GFF_ARGS);
+            else if (nct == 2) wmm_gradff_wave<8, 2, true>(CGNET_GFF_ARGS);
+            else if (nct == 3) wmm_gradff_wave<8, 3, true>(CGNET_GFF_ARGS);
+            else wmm_gradff_wave<8, 3, false>(CGNET_GFF_ARGS);
             break;
     }
 #undef CGNET_GFF_ARGS
@@ -853,7 +877,7 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
         p->gff_lds = std::max(p->gff_lds, (size_t)8 * d.tO * d.M);
     }
     // the matrix-core gradient kernel keeps a tile and two operand buffers per wave inside 64 KB of LDS
-    if (4 * ((size_t)p->gff_out_cap + 2 * (size_t)p->gff_go_cap) > 64 * 1024) p->gff_mfma = false;
+    if ((size_t)p->gff_out_cap + 2 * (size_t)p->gff_go_cap > 64 * 1024) p->gff_mfma = false;
     CGNET_REQUIRE(p->gff_lds <= 64 * 1024, CGNET_ERR_UNSUPPORTED, "t_O*(2l+1) too large for the gradient kernel");
     // heavier forward units first
     std::stable_sort(p->fwd_units.begin(), p->fwd_units.end(), [&](const WmmFwdUnit& a, const WmmFwdUnit& b) {
@@ -1074,9 +1098,9 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             const int groups = std::max(1, std::min(B, 8));
             const int spg = (B + groups - 1) / groups;
             const int out_bytes = plan->gff_out_cap, go_bytes = plan->gff_go_cap;   // per wave
-            const size_t lds = 4 * ((size_t)out_bytes + 2 * (size_t)go_bytes);
+            const size_t lds = (size_t)out_bytes + 2 * (size_t)go_bytes;
             CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)plan->gw_units_rc0.size(), (B + spg - 1) / spg),
-                         dim3(kThreads), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
+                         dim3(64), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
                          plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, out_bytes, go_bytes);
             CGNET_HIP(hipGetLastError());
             if (!plan->gff_zero_units.empty()) {
