@@ -241,7 +241,7 @@ __host__ __device__ inline size_t fwd_task_lds(const CgTask& t) {
 template <int TI, int TJ>
 __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restrict__ F, float2* __restrict__ FF,
                                           const float* __restrict__ CG, int nF, int nFF, int B,
-                                          int samples_per_group, double* __restrict__ stats_part, int sumT,
+                                          int samples_per_group, int group, double* __restrict__ stats_part, int sumT,
                                           unsigned char* smem) {
     const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
     const int nch = t.rows * t.tau2;
@@ -273,7 +273,7 @@ __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restr
     if (single && tid < nitems) fwd_item_setup<TI, TJ>(t, tid, cg, f1_0, f2_0, mine);
 
     double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};
-    const int b0 = blockIdx.y * samples_per_group;
+    const int b0 = group * samples_per_group;
     const int b1 = min(B, b0 + samples_per_group);
     if (b0 < b1) issue(b0, 0);
     for (int e = tid; e < ncg; e += kThreads) cg[e] = CG[t.cg_off + e];
@@ -329,7 +329,7 @@ __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restr
         for (int k = 0; k < 4; ++k) {
             const int ch = tid + kThreads * k;
             if (ch < nch) {
-                double* p = stats_part + ((size_t)blockIdx.y * sumT + t.chan0 + ch) * 2;
+                double* p = stats_part + ((size_t)group * sumT + t.chan0 + ch) * 2;
                 p[0] = s1[k];
                 p[1] = s2[k];
             }
@@ -342,15 +342,17 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
                   const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
                   double* __restrict__ stats_part, int sumT) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const CgTask t = tasks[blockIdx.x];
+    const UnitPart up = part_major((B + samples_per_group - 1) / samples_per_group);
+    const CgTask t = tasks[up.unit];
+    const int group = up.part;
 #define CGNET_FWD(TI_, TJ_) \
-    case (TI_) * 8 + (TJ_): fwd_group<TI_, TJ_>(t, F, FF, CG, nF, nFF, B, samples_per_group, stats_part, sumT, smem); break;
+    case (TI_) * 8 + (TJ_): fwd_group<TI_, TJ_>(t, F, FF, CG, nF, nFF, B, samples_per_group, group, stats_part, sumT, smem); break;
     switch (min(t.TI, 4) * 8 + min(t.TJ, 4)) {
         CGNET_FWD(1, 1) CGNET_FWD(1, 2) CGNET_FWD(1, 3) CGNET_FWD(1, 4)
         CGNET_FWD(2, 1) CGNET_FWD(2, 2) CGNET_FWD(2, 3) CGNET_FWD(2, 4)
         CGNET_FWD(3, 1) CGNET_FWD(3, 2) CGNET_FWD(3, 3) CGNET_FWD(3, 4)
         CGNET_FWD(4, 1) CGNET_FWD(4, 2) CGNET_FWD(4, 3)
-        default: fwd_group<4, 4>(t, F, FF, CG, nF, nFF, B, samples_per_group, stats_part, sumT, smem); break;
+        default: fwd_group<4, 4>(t, F, FF, CG, nF, nFF, B, samples_per_group, group, stats_part, sumT, smem); break;
     }
 #undef CGNET_FWD
 }
@@ -890,10 +892,11 @@ __global__ void __launch_bounds__(kThreads, 4)
 cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
                         const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                         const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
-                        int nF, int nFp, int nFF, int P2, int f1cap, int f2cap, int cgcap, int tcap) {
+                        int nF, int nFp, int nFF, int P2, int f1cap, int f2cap, int cgcap, int tcap, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const BwdUnit u = units[blockIdx.x];
-    const int b = blockIdx.y;
+    const UnitPart up = unit_major(B);
+    const BwdUnit u = units[up.unit];
+    const int b = up.part;
     const int tid = threadIdx.x, wave = tid >> 6;
     const int M1 = 2 * u.l1 + 1;
     const bool roleA = wave < u.nA;                  // wave-uniform
@@ -1447,8 +1450,9 @@ static int launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF,
     const int ntasks = (int)p->fwd_tasks.size();
     if (ntasks == 0 || B == 0) return CGNET_OK;
     const int ngroups = (B + spg - 1) / spg;
-    CGNET_REQUIRE(ngroups <= 65535, CGNET_ERR_UNSUPPORTED, "batch of %d needs %d sample groups (limit 65535)", B, ngroups);
-    CGNET_LAUNCH(cg_forward_kernel, dim3(ntasks, ngroups), dim3(kThreads), p->fwd_lds, s,
+    CGNET_REQUIRE((long long)ntasks * ngroups < (1LL << 31), CGNET_ERR_UNSUPPORTED,
+                  "%d tasks x %d sample groups exceed the grid limit", ntasks, ngroups);
+    CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(ntasks * ngroups)), dim3(kThreads), p->fwd_lds, s,
                        (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks, p->nF, p->nFF, B, spg, d_part, p->sumT);
     CGNET_HIP(hipGetLastError());
     return CGNET_OK;
@@ -1543,10 +1547,12 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
         CGNET_LAUNCH(cg_backward_pad_kernel, dim3((unsigned)(nbF + plan->nllls)), dim3(256), 0, s,
                      (const float2*)d_F, d_CG, Fp, CGP, plan->d_bwd_padmeta, plan->L, plan->nF, plan->bwd_nFp, B, nbF);
         CGNET_HIP(hipGetLastError());
-        CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)plan->bwd_units.size(), B), dim3(kThreads),
+        CGNET_REQUIRE((long long)B * (long long)plan->bwd_units.size() < (1LL << 31), CGNET_ERR_UNSUPPORTED,
+                      "%d samples x %zu units exceed the grid limit", B, plan->bwd_units.size());
+        CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kThreads),
                      plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
                      plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
-                     plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap);
+                     plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
         CGNET_HIP(hipGetLastError());
         const size_t n = (size_t)plan->nF * B;
         CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,

@@ -109,6 +109,30 @@ __device__ __forceinline__ void dma8(const void* __restrict__ src, void* dst, in
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(src) + 4 * tid, (lds_void_ptr)dst, 4, 0, 0);
 }
 
+// Grids over (unit, part) pairs -- a unit is a task or a run of channels, a part a sample or a group
+// of samples -- are launched one-dimensional and unit-major: all parts of the first unit, then all
+// parts of the second ...  With the units sorted longest first every long unit is under way before
+// any short one starts, and the grid drains through short work-groups.
+struct UnitPart { int unit, part; };
+__device__ __forceinline__ UnitPart unit_major(int nparts) {
+    UnitPart r;
+    r.unit = (int)(blockIdx.x / (unsigned)nparts);
+    r.part = (int)(blockIdx.x - (unsigned)r.unit * (unsigned)nparts);
+    return r;
+}
+
+// The other order: all units of the first part, then all units of the second ...  Work-groups that
+// run at the same time then stream neighbouring channel runs of the same samples, which spreads
+// their traffic evenly over the memory channels (the same run of many samples lies a whole sample
+// apart).  The kernels bound by memory use this one, the one bound by arithmetic the one above.
+__device__ __forceinline__ UnitPart part_major(int nparts) {
+    const unsigned nunits = gridDim.x / (unsigned)nparts;
+    UnitPart r;
+    r.part = (int)(blockIdx.x / nunits);
+    r.unit = (int)(blockIdx.x - (unsigned)r.part * nunits);
+    return r;
+}
+
 // 16-byte store of data that is not read again soon: marked non-temporal, so a long output stream
 // does not push the (small, re-read) operands of the kernel out of the L2 cache.
 __device__ __forceinline__ void stream_store16(void* dst, float a, float b, float c, float d) {

@@ -84,12 +84,13 @@ fn_stats_kernel(const float2* __restrict__ FF, const WmmDeg* __restrict__ degs,
                 double* __restrict__ part, int sumT) {
     extern __shared__ __align__(16) unsigned char smem[];
     float2* tile = reinterpret_cast<float2*>(smem);
-    const WmmChanUnit u = units[blockIdx.x];
+    const UnitPart up = part_major((B + samples_per_group - 1) / samples_per_group);
+    const WmmChanUnit u = units[up.unit];
     const WmmDeg d = degs[u.deg];
     const int n = u.nc * d.M;
     const int tid = threadIdx.x;
     double s1 = 0., s2 = 0.;
-    const int b0 = blockIdx.y * samples_per_group, b1 = min(B, b0 + samples_per_group);
+    const int b0 = up.part * samples_per_group, b1 = min(B, b0 + samples_per_group);
     for (int b = b0; b < b1; ++b) {
         const float2* src = FF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * d.M;
         for (int e = tid; e < n; e += kThreads) tile[e] = src[e];
@@ -107,7 +108,7 @@ fn_stats_kernel(const float2* __restrict__ FF, const WmmDeg* __restrict__ degs,
         __syncthreads();
     }
     if (tid < u.nc) {
-        double* p = part + ((size_t)blockIdx.y * sumT + d.cumT + u.c0 + tid) * 2;
+        double* p = part + ((size_t)up.part * sumT + d.cumT + u.c0 + tid) * 2;
         p[0] = s1;
         p[1] = s2;
     }
@@ -369,13 +370,14 @@ template <int TMAX>
 __global__ void __launch_bounds__(kThreads)
 wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, float2* __restrict__ out,
                    const WmmDeg* __restrict__ degs, const WmmFwdUnit* __restrict__ units, int B, int nFF, int nO,
-                   int stage_bytes, int depth) {
+                   int stage_bytes, int depth, int nparts) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const WmmFwdUnit u = units[blockIdx.x];
+    const UnitPart up = part_major(nparts);
+    const WmmFwdUnit u = units[up.unit];
     const WmmDeg d = degs[u.deg];
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave index, held in a scalar register
-    const int b_first = (blockIdx.y * 4 + w) * d.G;
+    const int b_first = (up.part * 4 + w) * d.G;
     if (b_first >= B) return;                                     // wave-uniform; the kernel has no barrier
     unsigned char* ring = smem + (size_t)w * depth * stage_bytes;
 #define CGNET_FWD_T(T_) wmm_forward_wave<T_>(FF, Wp, out, d, u, B, nFF, nO, b_first, ring, depth, stage_bytes, lane)
@@ -396,9 +398,9 @@ wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, 
 }
 
 template __global__ void wmm_forward_kernel<3>(const float2*, const float*, float2*, const WmmDeg*, const WmmFwdUnit*, int,
-                                               int, int, int, int);
+                                               int, int, int, int, int);
 template __global__ void wmm_forward_kernel<6>(const float2*, const float*, float2*, const WmmDeg*, const WmmFwdUnit*, int,
-                                               int, int, int, int);
+                                               int, int, int, int, int);
 
 // O = sum over k-slices of the partial outputs, in slice order
 __global__ void __launch_bounds__(256)
@@ -420,12 +422,12 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
 }
 
 // --------------------------------------------------------------------------- grad W (MFMA)
-// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples (blockIdx.y)
+// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples
 // into part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
 constexpr int kGwFFRegs = 4;    // 4 x 256 x 16 B = 16 KB of FF per sample and work-group
 constexpr int kGwGORegs = 3;    // 3 x 256 x 16 B = 12 KB of gO rows (16 rows of up to 95 complex)
 
-// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples (blockIdx.y)
+// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples
 // into part[chunk][nW].  Per sample the group's FF rows (nc channels x M, one contiguous run) and
 // the 16 gO rows are streamed through LDS with 16-byte lane-contiguous loads, double buffered;
 // each wave then reads its 16 channel rows in matrix-core operand order.
@@ -436,7 +438,8 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
     extern __shared__ __align__(16) unsigned char smem[];
     float2* ffbuf = reinterpret_cast<float2*>(smem);              // [2][ff_cap]
     float2* gobuf = ffbuf + 2 * ff_cap;                           // [2][go_cap]
-    const WmmChanUnit u = units[blockIdx.x];
+    const UnitPart up = part_major((B + samples_per_chunk - 1) / samples_per_chunk);
+    const WmmChanUnit u = units[up.unit];
     const WmmDeg d = degs[u.deg];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int i = lane & 15, kk = lane >> 4;
@@ -450,7 +453,7 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
     const int nblk = (M + 7) >> 3;
     const int n_ff = u.nc * M, n_go = go_rows * M;
     const size_t tot_ff = (size_t)B * nFF, tot_go = (size_t)B * nO;
-    const int b_begin = blockIdx.y * samples_per_chunk;
+    const int b_begin = up.part * samples_per_chunk;
     const int b_end = min(B, b_begin + samples_per_chunk);
 
     Run16<kGwFFRegs> pf;
@@ -501,7 +504,7 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
     }
     mfma_drain();
     if (cok) {
-        float2* dst = part + (size_t)blockIdx.y * nW;
+        float2* dst = part + (size_t)up.part * nW;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int to = u.rc * 16 + 4 * kk + v;
@@ -537,12 +540,13 @@ wmm_gradw_finish_kernel(const float2* __restrict__ part, const float* __restrict
 // gFF[b, c, m] = sum_to WT[c][to] * gO[b, to, m]   with WT = conj(W)/div packed channel-major
 __global__ void __launch_bounds__(kThreads)
 wmm_gradff_kernel(const float2* __restrict__ gO, const float2* __restrict__ WT, float2* __restrict__ gFF,
-                  const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int nFF, int nO) {
+                  const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int nFF, int nO, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
     float2* go = reinterpret_cast<float2*>(smem);      // [tO][M]
-    const WmmChanUnit u = units[blockIdx.x];
+    const UnitPart up = part_major(B);
+    const WmmChanUnit u = units[up.unit];
     const WmmDeg d = degs[u.deg];
-    const int b = blockIdx.y;
+    const int b = up.part;
     const int M = d.M, tO = d.tO;
     const float2* src = gO + (size_t)b * nO + d.cumO;
     for (int e = threadIdx.x; e < tO * M; e += kThreads) go[e] = src[e];
@@ -607,7 +611,7 @@ template <int NKS, int NT, bool ONE>
 __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, const float* __restrict__ Ap,
                                                 float2* __restrict__ gFF, const WmmDeg& d, const WmmChanUnit& u, int B,
                                                 int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes,
-                                                unsigned char* mine, int lane) {
+                                                unsigned char* mine, int lane, int group) {
     float* ol = reinterpret_cast<float*>(mine);                              // [16][2M]
     unsigned char* gobuf = mine + out_bytes;                                  // [2][go_bytes]
     const int i = lane & 15, kk = lane >> 4;
@@ -625,7 +629,7 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
     const float cx = (r == sel) ? (r ? -1.f : 1.f) : 0.f, cy = (r == sel) ? 0.f : 1.f;   // B = cx * re + cy * im
     const int nct = (2 * M + 15) >> 4;
     const int n_go = tO * M;                      // complex entries of the gO rows
-    const int b_begin = blockIdx.y * samples_per_group, b_end = min(B, b_begin + samples_per_group);
+    const int b_begin = group * samples_per_group, b_end = min(B, b_begin + samples_per_group);
     if (b_begin >= b_end) return;
     {
         // rows past t_O are read (times zero weights): they must hold finite values
@@ -723,10 +727,11 @@ wmm_gradff_mfma_kernel(const float2* __restrict__ gO, const float* __restrict__ 
                        const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
                        int samples_per_group, int nFF, int nO, int out_bytes, int go_bytes) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const WmmChanUnit u = units[blockIdx.x];
+    const UnitPart up = part_major((B + samples_per_group - 1) / samples_per_group);
+    const WmmChanUnit u = units[up.unit];
     const WmmDeg d = degs[u.deg];
     const int lane = threadIdx.x;
-#define CGNET_GFF_ARGS gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, smem, lane
+#define CGNET_GFF_ARGS gO, Ap, gFF, d, u, B, samples_per_group, nFF, nO, out_bytes, go_bytes, smem, lane, up.part
 #define CGNET_GFF(N_)                                                                     \
     case N_:                                                                              \
         if (nct == 1) wmm_gradff_wave<N_, 1, true>(CGNET_GFF_ARGS);                       \
@@ -971,7 +976,7 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
             const int ng = stat_groups_for(B);
             const int spg = (B + ng - 1) / ng;
             const int ngroups = (B + spg - 1) / spg;
-            CGNET_LAUNCH(fn_stats_kernel, dim3((unsigned)plan->stat_units.size(), ngroups), dim3(kThreads),
+            CGNET_LAUNCH(fn_stats_kernel, dim3((unsigned)(plan->stat_units.size() * ngroups)), dim3(kThreads),
                                plan->stat_lds, s, (const float2*)d_FF, plan->d_degs, plan->d_stat_units, plan->nFF,
                                B, spg, (double*)(base + ws.part), plan->sumT);
             CGNET_HIP(hipGetLastError());
@@ -1017,15 +1022,16 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     CGNET_REQUIRE(depth >= 2, CGNET_ERR_UNSUPPORTED, "forward stage of %d bytes does not fit the LDS ring", plan->fwd_stage_cap);
     const size_t lds = 4 * (size_t)depth * plan->fwd_stage_cap;
     if (plan->fwd_units_small > 0) {
-        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3((unsigned)plan->fwd_units_small, ygroups), dim3(kThreads), lds, s,
+        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3((unsigned)(plan->fwd_units_small * ygroups)), dim3(kThreads), lds, s,
                      (const float2*)d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO,
-                     plan->fwd_stage_cap, depth);
+                     plan->fwd_stage_cap, depth, ygroups);
         CGNET_HIP(hipGetLastError());
     }
     if ((int)plan->fwd_units.size() > plan->fwd_units_small) {
-        CGNET_LAUNCH(wmm_forward_kernel<6>, dim3((unsigned)(plan->fwd_units.size() - plan->fwd_units_small), ygroups),
+        CGNET_LAUNCH(wmm_forward_kernel<6>, dim3((unsigned)((plan->fwd_units.size() - plan->fwd_units_small) * ygroups)),
                      dim3(kThreads), lds, s, (const float2*)d_FF, Wp, out, plan->d_degs,
-                     plan->d_fwd_units + plan->fwd_units_small, B, plan->nFF, plan->nO, plan->fwd_stage_cap, depth);
+                     plan->d_fwd_units + plan->fwd_units_small, B, plan->nFF, plan->nO, plan->fwd_stage_cap, depth,
+                     ygroups);
         CGNET_HIP(hipGetLastError());
     }
     if (plan->maxS > 1) {
@@ -1075,7 +1081,7 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
             const int nchunks = gradw_chunks(B);
             const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
-            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)plan->gw_units.size(), nchunks), dim3(kThreads), lds, s,
+            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)(plan->gw_units.size() * nchunks)), dim3(kThreads), lds, s,
                                (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
                                kGradWChunk, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
             CGNET_HIP(hipGetLastError());
@@ -1099,15 +1105,15 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             const int spg = (B + groups - 1) / groups;
             const int out_bytes = plan->gff_out_cap, go_bytes = plan->gff_go_cap;   // per wave
             const size_t lds = (size_t)out_bytes + 2 * (size_t)go_bytes;
-            CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)plan->gw_units_rc0.size(), (B + spg - 1) / spg),
+            CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)(plan->gw_units_rc0.size() * ((B + spg - 1) / spg))),
                          dim3(64), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
                          plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, out_bytes, go_bytes);
             CGNET_HIP(hipGetLastError());
             if (!plan->gff_zero_units.empty()) {
                 // degrees that produce no output channels: the general kernel writes their zeros
-                CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_zero_units.size(), B), dim3(kThreads),
+                CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)(plan->gff_zero_units.size() * B)), dim3(kThreads),
                              plan->gff_lds, s, (const float2*)d_gO, (const float2*)nullptr, (float2*)d_gFF,
-                             plan->d_degs, plan->d_gff_zero_units, plan->nFF, plan->nO);
+                             plan->d_degs, plan->d_gff_zero_units, plan->nFF, plan->nO, B);
                 CGNET_HIP(hipGetLastError());
             }
         } else {
@@ -1116,9 +1122,9 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
                              (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
                 CGNET_HIP(hipGetLastError());
             }
-            CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)plan->gff_units.size(), B), dim3(kThreads),
+            CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)(plan->gff_units.size() * B)), dim3(kThreads),
                          plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
-                         plan->d_gff_units, plan->nFF, plan->nO);
+                         plan->d_gff_units, plan->nFF, plan->nO, B);
             CGNET_HIP(hipGetLastError());
         }
     }
