@@ -48,6 +48,8 @@ struct BwdUnit {
     int task_begin, task_end; // range in the unit-ordered task array (sorted by l2, then l)
     int nA;                   // waves that take slot 1; the other waves of the group take slot 2
     int TI, RW;               // slot-1 tiling: output rows per thread, lanes sharing one output
+    int p1off;                // slot-1 result: -1 = the unit's rows in the slot-1 area, else offset of its rows in the
+                              // slot-2 partial area (a degree whose task list is split over several units)
 };
 
 struct BwdUTask {
@@ -78,6 +80,7 @@ struct cgnet_cg_plan {
     int bwd_threads = 256;                       // work-group size of the backward kernel
     // register-resident backward (used when every unit fits; otherwise the LDS-accumulator kernel)
     bool bwd_fast = false;
+    bool bwd_hybrid = false;                     // units run cg_backward_hybrid_kernel (slot 2 on the matrix cores)
     std::vector<cgnet::BwdUnit> bwd_units;
     std::vector<cgnet::BwdUTask> bwd_utasks;
     cgnet::BwdUnit* d_bwd_units = nullptr;
@@ -101,6 +104,9 @@ constexpr int kBwdTileBytes = 14 * 1024;
 constexpr int kMaxTileChannels = 4 * kThreads;   // statistics: at most four channels per thread
 constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
+constexpr int kBwdPieces = 40;                   // unit backward: a unit holds at most this fraction of a sample's work
+constexpr size_t kMaxHybLds = 80 * 1024;        // hybrid unit backward: two groups of eight waves per CU
+constexpr long long kHybTileBytes = 28 * 1024;
 constexpr size_t kMaxUnitLds = 64 * 1024;       // unit backward: LDS-direct copies address the first 64 KB
 
 
@@ -793,19 +799,21 @@ struct BwdCtx {
 
 // Starts the copies of task t: tile and table into buffer `par`, the l2 slab (first task of a
 // run only) into slab buffer `f2par`.
+template <int NT>
 __device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, const BwdUTask& t, int par, int f2par) {
     const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
     const int ntile = u.rows * t.tau2 * M;
     char* tile = c.tile + par * (c.tcap + 16);
-    dma16<kThreads>(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
+    dma16<NT>(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
     if (ntile & 1) dma8(c.Gb + t.offFF + (ntile - 1), tile + 8 * (size_t)(ntile - 1), c.tid);
-    dma16<kThreads>(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
-    if (t.first_of_l2) dma16<kThreads>(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
+    dma16<NT>(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
+    if (t.first_of_l2) dma16<NT>(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
 }
 
 // Per-task prologue of both roles.  On entry `t` is the task whose copies were started one
 // task earlier into buffer `par`; on exit they are visible, `cur` holds that task and the
 // copies of the following task are in flight.  One barrier per task, executed by every thread.
+template <int NT>
 __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int ti, BwdUTask& t, BwdUTask& cur,
                                           int& par, int& f2par, const float*& cgp, const float2*& g,
                                           const float2*& f2) {
@@ -819,12 +827,12 @@ __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int
     if (ti + 1 < u.task_end) {
         t = c.tasks[ti + 1];
         if (t.first_of_l2) f2par ^= 1;
-        bwd_issue(c, u, t, par, f2par);
+        bwd_issue<NT>(c, u, t, par, f2par);
     }
 }
 
 // Waves of role A: gradient of slot 1 (rows of degree l1), kept in registers for the whole unit.
-template <int TI, int RW>
+template <int NT, int TI, int RW>
 __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdUTask t,
                                                 float2* __restrict__ dst) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
@@ -838,7 +846,7 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         BwdUTask cur;
         const float* cgp;
         const float2 *g, *f2;
-        bwd_stage(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        bwd_stage<NT>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
         bwd_accum<1, TI, RW>(q, cgp, g, f2, c.rtid, ax, ay);
         if (cur.last_of_l2) {
@@ -867,7 +875,7 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
         BwdUTask cur;
         const float* cgp;
         const float2 *g, *f2;
-        bwd_stage(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        bwd_stage<kThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
 #define CGNET_CALL_B(TI_, RW_) bwd_accum<2, TI_, RW_>(q, cgp, g, c.f1, c.rtid, ax, ay)
         CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_CALL_B)
@@ -921,16 +929,174 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
     __syncthreads();                                 // the clearing stores precede every copy
     const BwdUTask t0 = tasks[u.task_begin];
     dma16<kThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
-    bwd_issue(c, u, t0, 0, 0);
+    bwd_issue<kThreads>(c, u, t0, 0, 0);
 
     // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
-        float2* dst = part1 + (size_t)b * nF + u.offF1;
-#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<TI_, RW_>(c, u, t0, dst)
+        float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
+#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<kThreads, TI_, RW_>(c, u, t0, dst)
         CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
         bwd_unit_loop_b(c, u, t0, part2 + (size_t)b * P2);
+    }
+}
+
+// ---- unit backward, slot 2 on the matrix cores ----------------------------------------------
+// For a fixed m of the tile, G_m = gFF[t1, t2, m] is a rows x tau2 complex matrix and
+//   gF2[t2, m2] += sum_t1 G_m[t1, t2] * (C[m][m2] conj F1[t1][m - m2])       (tau2 x rows)(rows x window of m2)
+// is a small matrix product: rows of the accumulator = the up to 16 channels of degree l2, columns
+// = up to two tiles of 16 values of m2, reduction over the up to 16 rows of the unit in steps of 4.
+// Work-groups of eight waves: waves 0-3 keep the slot-1 gradient on the vector ALUs exactly as in
+// cg_backward_unit_kernel, waves 4-7 take slot 2 here, each every fourth m.  The two halves use
+// different pipelines of the same SIMDs (a wave of either half on each), so the vector ALUs carry
+// about half the arithmetic.  The four partial slot-2 gradients leave as separate slabs;
+// cg_backward_combine_kernel adds them.
+constexpr int kHybThreads = 512;
+constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
+                                    // slot-2 gradient) slot 2 on the matrix cores
+constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
+
+template <int NK>
+__device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
+                                            const float2* __restrict__ g, const float2* __restrict__ f1, int part,
+                                            int split, int lane, f32x4 (&dre)[2], f32x4 (&dim)[2]) {
+    const int l = q.l, l1 = q.l1, l2 = q.l2;
+    const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
+    const int rows = q.rows, tau2 = q.tau2;
+    const int ntiles = (M2 + 15) >> 4;
+    const int i = lane & 15, kk = lane >> 4;
+    const int io = min(i, tau2 - 1);                              // rows past the last channel repeat it (never stored)
+    // per reduction step: the lane's row of the unit, its tile entry and fragment row
+    int goff[NK], foff[NK];
+    bool kval[NK];
+#pragma unroll
+    for (int c = 0; c < NK; ++c) {
+        const int k = 4 * c + kk;
+        const int kc = min(k, rows - 1);
+        kval[c] = k < rows;
+        goff[c] = (kc * tau2 + io) * M;
+        foff[c] = kc * (M1 + 1);
+    }
+    for (int mi = part; mi < M; mi += split) {
+        const int m = mi - l;
+        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);    // valid m2
+        if (hi < lo) continue;
+        float2 gq[NK];
+#pragma unroll
+        for (int c = 0; c < NK; ++c) gq[c] = g[goff[c] + mi];
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile) {
+            if (tile >= ntiles || hi + l2 < 16 * tile || lo + l2 > 16 * tile + 15) continue;    // wave-uniform
+            const int m2 = 16 * tile + i - l2;                    // this lane's column
+            const bool cval = m2 >= lo && m2 <= hi;
+            const int m2c = min(max(m2, lo), hi);
+            const float cc = cgp[(kTabLo + mi) * M2 + m2c + l2];
+            const float cv = cval ? cc : 0.f;
+            const int fcol = m - m2c + l1;                        // column of the slot-1 fragment
+            float2 fq[NK];
+#pragma unroll
+            for (int c = 0; c < NK; ++c) fq[c] = f1[foff[c] + fcol];
+#pragma unroll
+            for (int c = 0; c < NK; ++c) {
+                const float w = kval[c] ? cv : 0.f;
+                const float bx = w * fq[c].x, by = -w * fq[c].y;  // C conj(f)
+                dre[tile] = mfma4(gq[c].x, bx, dre[tile]);
+                dim[tile] = mfma4(gq[c].x, by, dim[tile]);
+                dre[tile] = mfma4(-gq[c].y, by, dre[tile]);
+                dim[tile] = mfma4(gq[c].y, bx, dim[tile]);
+            }
+        }
+    }
+}
+
+// Stores the wave's accumulator tiles: rows = channels, columns of an m axis of length Mo.
+__device__ __forceinline__ void bwd_mm_store(const f32x4 (&dre)[2], const f32x4 (&dim)[2], int n_out, int Mo, int lane,
+                                             float2* __restrict__ dst) {
+    const int j = lane & 15, kk = lane >> 4;
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+        const int col = 16 * tile + j;
+        if (col < Mo) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int ch = 4 * kk + v;
+                if (ch < n_out) dst[ch * Mo + col] = make_float2(dre[tile][v], dim[tile][v]);
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit& u, BwdUTask t, int part, int split,
+                                                  int lane, float2* __restrict__ part2_b) {
+    f32x4 dre[2], dim[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    int par = 0, f2par = 0;
+    for (int ti = u.task_begin; ti < u.task_end; ++ti) {
+        BwdUTask cur;
+        const float* cgp;
+        const float2 *g, *f2;
+        bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+        switch ((u.rows + 3) >> 2) {
+            case 1: bwd_mm_task<1>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
+            case 2: bwd_mm_task<2>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
+            case 3: bwd_mm_task<3>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
+            default: bwd_mm_task<4>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
+        }
+        if (cur.last_of_l2) {
+            const int M2 = 2 * cur.l2 + 1;
+            mfma_drain();
+            bwd_mm_store(dre, dim, cur.tau2, M2, lane, part2_b + cur.p2off + (size_t)part * cur.tau2 * M2);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kHybThreads, 4)
+cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
+                          const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
+                          const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
+                          int nF, int nFp, int nFF, int P2, int f1cap, int f2cap, int cgcap, int tcap, int B) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const UnitPart up = unit_major(B);
+    const BwdUnit u = units[up.unit];
+    const int b = up.part;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M1 = 2 * u.l1 + 1;
+    const bool roleA = wave < u.nA;                  // wave-uniform
+    BwdCtx c;
+    c.Fp = Fp + (size_t)b * nFp;
+    c.Gb = gFF + (size_t)b * nFF;
+    c.CGP = CGP;
+    c.tasks = tasks;
+    c.f1 = reinterpret_cast<float2*>(smem + 16);
+    c.f2 = reinterpret_cast<char*>(smem) + 16 + f1cap;
+    c.cg = c.f2 + 2 * f2cap;
+    c.tile = c.cg + 2 * cgcap + 16;
+    c.f2cap = f2cap; c.cgcap = cgcap; c.tcap = tcap;
+    c.tid = tid;
+    c.rtid = tid;                                    // role A: threads 0 .. 64 * nA - 1
+    {
+        const int n16 = (int)(bwd_unit_lds(f1cap, f2cap, cgcap, tcap) >> 4);
+        float4* z = reinterpret_cast<float4*>(smem);
+        for (int e = tid; e < n16; e += kHybThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __syncthreads();                                 // the clearing stores precede every copy
+    const BwdUTask t0 = tasks[u.task_begin];
+    dma16<kHybThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
+    bwd_issue<kHybThreads>(c, u, t0, 0, 0);
+    // The two roles run the same sequence of barriers (one per task) from different code paths.
+    if (roleA) {
+        float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
+#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<kHybThreads, TI_, RW_>(c, u, t0, dst)
+        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#undef CGNET_LOOP_A
+    } else {
+        bwd_hybrid_loop_b(c, u, t0, wave - u.nA, kHybWaves - u.nA, tid & 63, part2 + (size_t)b * P2);
     }
 }
 
@@ -1221,7 +1387,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
 
     // ---- register-resident backward: units = (l1, range of t1 rows), tasks ordered by (l2, l)
     std::vector<int> combine_meta, pad_meta;
-    {
+    // first with slot 2 on the matrix cores where the shapes allow it, then all on the vector ALUs
+    for (int attempt = 0; attempt < 2 && !p->bwd_fast; ++attempt) {
         bool ok = true;
         int P2 = 0;
         size_t lds_max = 0;
@@ -1233,10 +1400,18 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             if ((long long)cgp_off[i] + len > INT32_MAX) { ok = false; break; }
             cgp_off[i + 1] = cgp_off[i] + (int)len;
         }
+        // Slot 2 on the matrix cores: needs every channel count to fit one 16-row tile (and to fill a
+        // good part of it), the m2 axis two 16-column tiles.  CGNET_BWD_HYBRID=0 keeps all on the vector ALUs.
+        bool hybrid = attempt == 0 && n1 - 1 <= 15;
+        for (int l = 0; l < n1; ++l)
+            if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) hybrid = false;
+        if (const char* e = getenv("CGNET_BWD_HYBRID"); e && e[0] == '0') hybrid = false;
+        if (attempt == 0 && !hybrid) continue;
+        const long long tile_limit = hybrid ? kHybTileBytes : kBwdTileBytes;
         int f1cap = 0, f2cap = 0, cgcap = 0, tcap = 0;
         std::vector<int> own1(n1, 0);
         std::vector<std::vector<int>> lam_offs(n1);
-        std::vector<double> unit_cost;
+        std::vector<double> unit_cost, task_cost;
         for (int l1 = 0; l1 < n1 && ok; ++l1) {
             std::vector<int> tri;
             for (int i = 0; i < nllls; ++i)
@@ -1248,7 +1423,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             });
             const int tau1 = h_t_F[l1], M1 = 2 * l1 + 1;
             const int nt = (int)tri.size();
-            struct Choice { double total = -1; int rows = 0, nA = 0, TI = 0, RW = 0; std::vector<int> bTI, bRW; };
+            struct Choice { double total = -1; int rows = 0, nA = 0, TI = 0, RW = 0; std::vector<int> bTI, bRW; std::vector<double> tcost; };
             Choice best;
             int prev_rows = -1;
             for (int nchunks = 1; nchunks <= tau1; ++nchunks) {
@@ -1257,10 +1432,11 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 prev_rows = rows_c;
                 long long max_tile = 0;
                 for (int i : tri) max_tile = std::max(max_tile, 8LL * rows_c * h_t_F[tl2[i]] * (2 * tl[i] + 1));
-                if (max_tile > kBwdTileBytes && rows_c > 1) continue;
+                if (max_tile > tile_limit && rows_c > 1) continue;
+                if (hybrid && rows_c > kHybMaxRows) continue;
                 const int real_chunks = (tau1 + rows_c - 1) / rows_c;
-                for (int nA = 1; nA <= 3; ++nA) {
-                    const int lanesA = 64 * nA, lanesB = kThreads - lanesA;
+                for (int nA = hybrid ? 4 : 1; nA <= (hybrid ? 6 : 3); ++nA) {
+                    const int lanesA = 64 * nA, lanesB = hybrid ? 0 : kThreads - lanesA;
                     // slot 2: best tiling per task (constant within a run of equal l2)
                     std::vector<double> costB(nt);
                     std::vector<int> bTI(nt), bRW(nt);
@@ -1268,7 +1444,14 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     for (int k = 0; k < nt && feasible; ++k) {
                         const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
                         double bc = -1;
-                        for (int ti = 1; ti <= kBwdMaxTI; ++ti)
+                        if (hybrid) {
+                            // a matrix instruction occupies its pipeline for eight vector-instruction slots
+                            const int Mq = 2 * tl[tri[k]] + 1;
+                            const int split = kHybWaves - nA;
+                            bc = ((Mq + split - 1) / split) * (double)((M2 + 15) / 16) * (((rows_c + 3) / 4) * 32.0 + 26.0);
+                            bTI[k] = 1; bRW[k] = 1;
+                        }
+                        for (int ti = 1; ti <= kBwdMaxTI && !hybrid; ++ti)
                             for (int rw = 1; rw <= 16; rw *= 2) {
                                 if (rw > 1 && rw / 2 >= rows_c) continue;
                                 const int items = ((tau2 + ti - 1) / ti) * ((M2 + 1) / 2);
@@ -1288,16 +1471,18 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                             const int items = ((rows_c + ti - 1) / ti) * ((M1 + 1) / 2);
                             if (items * rw > lanesA) continue;
                             double total = 0;
+                            std::vector<double> tcost(nt);
                             for (int k = 0; k < nt; ++k) {
                                 const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
                                 const double cA = ((tau2 + rw - 1) / rw) * (double)M2 * (8.0 * ti + 14.0);
                                 const double stage = 12.0 * rows_c * tau2 * (2 * tl[tri[k]] + 4) / kThreads + 200.0;
-                                total += std::max(cA, costB[k]) + stage;
+                                tcost[k] = std::max(cA, costB[k]) + stage;
+                                total += tcost[k];
                             }
                             total *= real_chunks;
                             if (best.total < 0 || total < best.total) {
                                 best.total = total; best.rows = rows_c; best.nA = nA; best.TI = ti; best.RW = rw;
-                                best.bTI = bTI; best.bRW = bRW;
+                                best.bTI = bTI; best.bRW = bRW; best.tcost = tcost;
                             }
                         }
                 }
@@ -1311,6 +1496,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 u.offF1p = cumFp[l1] + r0 * (M1 + 1);
                 u.task_begin = (int)p->bwd_utasks.size();
                 u.nA = best.nA; u.TI = best.TI; u.RW = best.RW;
+                u.p1off = -1;
                 f1cap = std::max(f1cap, (int)align_up((size_t)8 * u.rows * (M1 + 1), 16));
                 for (int k = 0; k < nt; ++k) {
                     const int i = tri[k];
@@ -1326,14 +1512,18 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     t.first_of_l2 = (k == 0 || tl2[tri[k - 1]] != t.l2) ? 1 : 0;
                     t.last_of_l2 = (k + 1 == nt || tl2[tri[k + 1]] != t.l2) ? 1 : 0;
                     if (t.first_of_l2) {
-                        lam_offs[t.l2].push_back(P2);
+                        // one slab per (unit, l2); the matrix-core waves write one each
                         t.p2off = P2;
-                        P2 += t.tau2 * M2;
+                        for (int sp = 0; sp < (hybrid ? kHybWaves - best.nA : 1); ++sp) {
+                            lam_offs[t.l2].push_back(P2);
+                            P2 += t.tau2 * M2;
+                        }
                     } else {
                         t.p2off = p->bwd_utasks.back().p2off;
                     }
                     t.TI = best.bTI[k]; t.RW = best.bRW[k];
                     p->bwd_utasks.push_back(t);
+                    task_cost.push_back(best.tcost[k]);
                     const size_t tile_bytes = align_up((size_t)8 * u.rows * t.tau2 * M, 16);
                     if (tile_bytes > kMaxLds) { ok = false; break; }
                     f2cap = std::max(f2cap, (int)align_up((size_t)8 * t.tau2 * (M2 + 1), 16));
@@ -1343,13 +1533,59 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 u.task_end = (int)p->bwd_utasks.size();
                 lds_max = bwd_unit_lds(f1cap, f2cap, cgcap, tcap);
                 p->bwd_units.push_back(u);
-                unit_cost.push_back(best.total);
             }
+        }
+        // A unit longer than its share of the machine would outlast all others: task lists are cut at
+        // the boundaries between runs of equal l2 into pieces of at most 1/kBwdPieces of a sample's work.
+        // The pieces after the first of a degree put their slot-1 result into slabs of the slot-2
+        // partial area (the same cuts for all row ranges of the degree, so every slab is covered).
+        if (ok) {
+            double all = 0;
+            for (double c : task_cost) all += c;
+            int pieces = kBwdPieces;
+            if (const char* e = getenv("CGNET_BWD_PIECES")) pieces = std::max(1, atoi(e));
+            const double target = all / pieces;
+            std::vector<BwdUnit> cut;
+            std::vector<int> slab_of_piece;              // per degree: slab offsets of pieces 1, 2, ...
+            int cur_l1 = -1;
+            for (const BwdUnit& u : p->bwd_units) {
+                const int M1 = 2 * u.l1 + 1, tau1 = h_t_F[u.l1];
+                const int r0 = (u.offF1 - p->cumF[u.l1]) / M1;
+                if (u.l1 != cur_l1) { cur_l1 = u.l1; slab_of_piece.clear(); }
+                double acc = 0, piece_cost = 0;
+                int start = u.task_begin, piece = 0;
+                // all row ranges of a degree have the same task list and costs, hence the same cuts
+                for (int k = u.task_begin; k < u.task_end; ++k) {
+                    acc += task_cost[k];
+                    piece_cost += task_cost[k];
+                    const bool last = k + 1 == u.task_end;
+                    if (last || (p->bwd_utasks[k].last_of_l2 && acc >= target)) {
+                        BwdUnit v = u;
+                        v.task_begin = start;
+                        v.task_end = k + 1;
+                        if (piece > 0) {
+                            if ((int)slab_of_piece.size() < piece) {
+                                slab_of_piece.push_back(P2);
+                                lam_offs[u.l1].push_back(P2);
+                                P2 += tau1 * M1;
+                            }
+                            v.p1off = slab_of_piece[piece - 1] + r0 * M1;
+                        }
+                        cut.push_back(v);
+                        unit_cost.push_back(piece_cost);
+                        start = k + 1;
+                        acc = piece_cost = 0;
+                        ++piece;
+                    }
+                }
+            }
+            p->bwd_units.swap(cut);
         }
         // CGNET_BWD_GENERAL=1 forces the LDS-accumulator kernel (kept for shapes the unit scheme cannot hold)
         const char* force_general = getenv("CGNET_BWD_GENERAL");
         if (force_general && force_general[0] == '1') ok = false;
-        if (ok && !p->bwd_units.empty() && lds_max <= kMaxUnitLds) {
+        if (ok && !p->bwd_units.empty() && lds_max <= (hybrid ? kMaxHybLds : kMaxUnitLds)) {
+            p->bwd_hybrid = hybrid;
             // longest units first
             std::vector<int> order(p->bwd_units.size());
             for (size_t k = 0; k < order.size(); ++k) order[k] = (int)k;
@@ -1369,8 +1605,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 pad_meta.insert(pad_meta.end(), v, v + 5);
             }
             if (const char* dbg = getenv("CGNET_DEBUG"); dbg && dbg[0] == '1') {
-                fprintf(stderr, "[cgnet] backward units=%zu tasks=%zu P2=%d lds=%zu\n", p->bwd_units.size(),
-                        p->bwd_utasks.size(), P2, lds_max);
+                fprintf(stderr, "[cgnet] backward units=%zu tasks=%zu P2=%d lds=%zu%s\n", p->bwd_units.size(),
+                        p->bwd_utasks.size(), P2, lds_max, hybrid ? " (slot 2 on the matrix cores)" : "");
                 for (const BwdUnit& u : p->bwd_units) {
                     const BwdUTask& t0 = p->bwd_utasks[u.task_begin];
                     const BwdUTask& t1 = p->bwd_utasks[u.task_end - 1];
@@ -1410,7 +1646,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         CGNET_HIP(hipMalloc((void**)&p->d_bwd_padmeta, sizeof(int) * pad_meta.size()));
         CGNET_HIP(hipMemcpy(p->d_bwd_padmeta, pad_meta.data(), sizeof(int) * pad_meta.size(), hipMemcpyHostToDevice));
         if (p->bwd_fast_lds > 64 * 1024)
-            CGNET_HIP(hipFuncSetAttribute((const void*)cg_backward_unit_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_fast_lds));
+            CGNET_HIP(hipFuncSetAttribute(p->bwd_hybrid ? (const void*)cg_backward_hybrid_kernel : (const void*)cg_backward_unit_kernel,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_fast_lds));
     }
     if (p->fwd_lds > 64 * 1024)
         CGNET_HIP(hipFuncSetAttribute((const void*)cg_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->fwd_lds));
@@ -1549,10 +1786,17 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
         CGNET_HIP(hipGetLastError());
         CGNET_REQUIRE((long long)B * (long long)plan->bwd_units.size() < (1LL << 31), CGNET_ERR_UNSUPPORTED,
                       "%d samples x %zu units exceed the grid limit", B, plan->bwd_units.size());
-        CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kThreads),
-                     plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
-                     plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
-                     plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
+        if (plan->bwd_hybrid) {
+            CGNET_LAUNCH(cg_backward_hybrid_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads),
+                         plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
+                         plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
+                         plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
+        } else {
+            CGNET_LAUNCH(cg_backward_unit_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kThreads),
+                         plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
+                         plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
+                         plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
+        }
         CGNET_HIP(hipGetLastError());
         const size_t n = (size_t)plan->nF * B;
         CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,

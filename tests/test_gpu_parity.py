@@ -567,6 +567,7 @@ def test_full_size_stack_config5_runs(dev):
     from cgnet_amd import CGNet
     lmax, bsz = 20, 32
     taus = [[1] * 21] + [[16] * 21] * 4
+    torch.manual_seed(5)                       # the layers and the head draw their initial weights from the global generator
     net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
     assert net.output_length == 2 * (1 + 4 * 16)
     g = torch.Generator().manual_seed(5)
@@ -595,9 +596,13 @@ def test_full_size_stack_config5_runs(dev):
     xe = x0.clone().requires_grad_(True)
     torch.nn.functional.cross_entropy(head(net(xe)), labels).backward()
     want = float((xe.grad.double() * d.double()).sum())
-    h = 1e-2
-    got = (f(x0 + h * d) - f(x0 - h * d)) / (2 * h)
-    assert got == pytest.approx(want, rel=5e-2, abs=1e-5)
+    # central differences at two step sizes, extrapolated (removes the h^2 term of the truncation error);
+    # the steps are long because the loss (tens) is evaluated in single precision: rounding noise / h must stay small
+    h = 1.0
+    d1 = (f(x0 + h * d) - f(x0 - h * d)) / (2 * h)
+    d2 = (f(x0 + 0.5 * h * d) - f(x0 - 0.5 * h * d)) / h
+    got = (4 * d2 - d1) / 3
+    assert got == pytest.approx(want, rel=5e-2, abs=2e-3)
 
 
 def test_classifier_from_coefficient_file(dev, tmp_path):
