@@ -567,7 +567,8 @@ def test_full_size_stack_config5_runs(dev):
     from cgnet_amd import CGNet
     lmax, bsz = 20, 32
     taus = [[1] * 21] + [[16] * 21] * 4
-    torch.manual_seed(5)                       # the layers and the head draw their initial weights from the global generator
+    torch.manual_seed(5)                       # the layers and the head draw their initial weights from the global generator,
+    np.random.seed(5)                          # the initial running stds from numpy's (as in the reference, CG_layers.py:116)
     net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
     assert net.output_length == 2 * (1 + 4 * 16)
     g = torch.Generator().manual_seed(5)
@@ -584,25 +585,29 @@ def test_full_size_stack_config5_runs(dev):
     for cg in net.cgs:
         assert torch.isfinite(cg.bnWMM.W.grad).all() and float(cg.bnWMM.W.grad.abs().max()) > 0
         assert cg.bnWMM.bn_cnt == 2.0
-    # directional derivative of the loss along a random input direction, evaluation mode (fixed statistics)
+    # Directional derivative, evaluation mode (fixed statistics), of a fixed linear functional of the
+    # embedding scaled to O(1) -- the cross-entropy of embeddings in the hundreds saturates and its
+    # single-precision rounding noise swamps a difference quotient.  Central differences at two step
+    # sizes, extrapolated (removes the h^2 term of the truncation error).
     net.eval()
     x0 = x.detach()
-    d = torch.randn_like(x0)
+    d = torch.randn(x0.shape, generator=g).to(dev)
     d /= d.norm()
+    with torch.no_grad():
+        e0 = net(x0)
+    r = torch.randn(e0.shape, generator=g).to(dev) / (e0.abs().mean(0, keepdim=True) + 1e-6) / e0.numel()
 
     def f(t):
         with torch.no_grad():
-            return float(torch.nn.functional.cross_entropy(head(net(t)).double(), labels))
+            return float((net(t).double() * r.double()).sum())
     xe = x0.clone().requires_grad_(True)
-    torch.nn.functional.cross_entropy(head(net(xe)), labels).backward()
+    (net(xe) * r).sum().backward()
     want = float((xe.grad.double() * d.double()).sum())
-    # central differences at two step sizes, extrapolated (removes the h^2 term of the truncation error);
-    # the steps are long because the loss (tens) is evaluated in single precision: rounding noise / h must stay small
     h = 1.0
     d1 = (f(x0 + h * d) - f(x0 - h * d)) / (2 * h)
     d2 = (f(x0 + 0.5 * h * d) - f(x0 - 0.5 * h * d)) / h
     got = (4 * d2 - d1) / 3
-    assert got == pytest.approx(want, rel=5e-2, abs=2e-3)
+    assert got == pytest.approx(want, rel=3e-2, abs=1e-7)
 
 
 def test_classifier_from_coefficient_file(dev, tmp_path):
