@@ -142,6 +142,7 @@ def main():
         "wmm_gradff_mfma_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
         "wmm_gradff_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
         "cg_backward_unit_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
+        "cg_backward_hybrid_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
     # HBM bytes per launch at this workload from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
