@@ -10,6 +10,7 @@ is no CPU implementation behind these classes.  Modules can be constructed witho
 (parameters and metadata only); the native plans are created on first use.
 """
 import functools
+import os
 
 import numpy as np
 import torch
@@ -313,6 +314,17 @@ class CG_woFilter_cuda(nn.Module):
 
 
 # --------------------------------------------------------------------------- the whole layer
+_OVERLAP_GRAD_W = int(os.environ.get("CGNET_OVERLAP_GW", "1"))
+_side_streams = {}
+
+
+def _side_stream(device):
+    key = torch.device(device).index
+    if key not in _side_streams:
+        _side_streams[key] = torch.cuda.Stream(device=device)
+    return _side_streams[key]
+
+
 class _CGBN_fused(torch.autograd.Function):
     """CG product -> fragment norm -> weight mixing in one autograd node.  Same arithmetic as
     ``_CG_sparse_cuda`` followed by ``_MyBatchNormWeightMM_cuda``; the only difference is that the
@@ -346,9 +358,24 @@ class _CGBN_fused(torch.autograd.Function):
         need_F, need_W = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         grad_FF = torch.empty_like(FF) if need_F else None
         grad_W = torch.empty_like(W) if need_W else None
+        grad_F = None
+        if need_F and need_W and _OVERLAP_GRAD_W:
+            # The weight gradient depends on nothing the other chain produces: it runs on a second
+            # stream (default priority) beside grad FF -> CG backward and is joined at the end.  What
+            # it gains comes from the overlap with the grad FF kernel (one reads FF, the other writes
+            # gFF); CGNET_OVERLAP_GW=0 keeps the whole backward on one stream.
+            main = torch.cuda.current_stream(Fs.device)
+            side = _side_stream(Fs.device)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
+            ctx.wmm_plan.backward(grad_output, grad_FF, None, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
+            grad_F = torch.empty_like(Fs)
+            ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
+            main.wait_stream(side)
+            return grad_F, grad_W, None, None, None, None, None, None, None
         if need_F or need_W:
             ctx.wmm_plan.backward(grad_output, grad_FF, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
-        grad_F = None
         if need_F:
             grad_F = torch.empty_like(Fs)
             ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
