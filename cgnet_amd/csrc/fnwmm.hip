@@ -793,6 +793,12 @@ static void free_plan(cgnet_wmm_plan* plan) {
     delete plan;
 }
 
+// Number of work-groups of a one-dimensional (unit, part) grid; 0 when the product exceeds the grid limit.
+static unsigned grid_1d(size_t nunits, size_t nparts) {
+    const unsigned long long n = (unsigned long long)nunits * nparts;
+    return n < (1ULL << 31) ? (unsigned)n : 0u;
+}
+
 extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_t_FF, const int* h_t_O) {
     clear_error();
     CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
@@ -976,7 +982,7 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
             const int ng = stat_groups_for(B);
             const int spg = (B + ng - 1) / ng;
             const int ngroups = (B + spg - 1) / spg;
-            CGNET_LAUNCH(fn_stats_kernel, dim3((unsigned)(plan->stat_units.size() * ngroups)), dim3(kThreads),
+            CGNET_LAUNCH(fn_stats_kernel, dim3(grid_1d(plan->stat_units.size(), ngroups)), dim3(kThreads),
                                plan->stat_lds, s, (const float2*)d_FF, plan->d_degs, plan->d_stat_units, plan->nFF,
                                B, spg, (double*)(base + ws.part), plan->sumT);
             CGNET_HIP(hipGetLastError());
@@ -1022,13 +1028,13 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     CGNET_REQUIRE(depth >= 2, CGNET_ERR_UNSUPPORTED, "forward stage of %d bytes does not fit the LDS ring", plan->fwd_stage_cap);
     const size_t lds = 4 * (size_t)depth * plan->fwd_stage_cap;
     if (plan->fwd_units_small > 0) {
-        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3((unsigned)(plan->fwd_units_small * ygroups)), dim3(kThreads), lds, s,
+        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3(grid_1d(plan->fwd_units_small, ygroups)), dim3(kThreads), lds, s,
                      (const float2*)d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO,
                      plan->fwd_stage_cap, depth, ygroups);
         CGNET_HIP(hipGetLastError());
     }
     if ((int)plan->fwd_units.size() > plan->fwd_units_small) {
-        CGNET_LAUNCH(wmm_forward_kernel<6>, dim3((unsigned)((plan->fwd_units.size() - plan->fwd_units_small) * ygroups)),
+        CGNET_LAUNCH(wmm_forward_kernel<6>, dim3(grid_1d(plan->fwd_units.size() - plan->fwd_units_small, ygroups)),
                      dim3(kThreads), lds, s, (const float2*)d_FF, Wp, out, plan->d_degs,
                      plan->d_fwd_units + plan->fwd_units_small, B, plan->nFF, plan->nO, plan->fwd_stage_cap, depth,
                      ygroups);
@@ -1081,7 +1087,7 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
             const int nchunks = gradw_chunks(B);
             const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
-            CGNET_LAUNCH(wmm_gradw_kernel, dim3((unsigned)(plan->gw_units.size() * nchunks)), dim3(kThreads), lds, s,
+            CGNET_LAUNCH(wmm_gradw_kernel, dim3(grid_1d(plan->gw_units.size(), nchunks)), dim3(kThreads), lds, s,
                                (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
                                kGradWChunk, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
             CGNET_HIP(hipGetLastError());
@@ -1105,13 +1111,13 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             const int spg = (B + groups - 1) / groups;
             const int out_bytes = plan->gff_out_cap, go_bytes = plan->gff_go_cap;   // per wave
             const size_t lds = (size_t)out_bytes + 2 * (size_t)go_bytes;
-            CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3((unsigned)(plan->gw_units_rc0.size() * ((B + spg - 1) / spg))),
+            CGNET_LAUNCH(wmm_gradff_mfma_kernel, dim3(grid_1d(plan->gw_units_rc0.size(), (B + spg - 1) / spg)),
                          dim3(64), lds, s, (const float2*)d_gO, (const float*)Ap, (float2*)d_gFF, plan->d_degs,
                          plan->d_gw_units_rc0, B, spg, plan->nFF, plan->nO, out_bytes, go_bytes);
             CGNET_HIP(hipGetLastError());
             if (!plan->gff_zero_units.empty()) {
                 // degrees that produce no output channels: the general kernel writes their zeros
-                CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)(plan->gff_zero_units.size() * B)), dim3(kThreads),
+                CGNET_LAUNCH(wmm_gradff_kernel, dim3(grid_1d(plan->gff_zero_units.size(), B)), dim3(kThreads),
                              plan->gff_lds, s, (const float2*)d_gO, (const float2*)nullptr, (float2*)d_gFF,
                              plan->d_degs, plan->d_gff_zero_units, plan->nFF, plan->nO, B);
                 CGNET_HIP(hipGetLastError());
@@ -1122,7 +1128,7 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
                              (const float2*)d_W, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, WT, plan->nW);
                 CGNET_HIP(hipGetLastError());
             }
-            CGNET_LAUNCH(wmm_gradff_kernel, dim3((unsigned)(plan->gff_units.size() * B)), dim3(kThreads),
+            CGNET_LAUNCH(wmm_gradff_kernel, dim3(grid_1d(plan->gff_units.size(), B)), dim3(kThreads),
                          plan->gff_lds, s, (const float2*)d_gO, (const float2*)WT, (float2*)d_gFF, plan->d_degs,
                          plan->d_gff_units, plan->nFF, plan->nO, B);
             CGNET_HIP(hipGetLastError());
