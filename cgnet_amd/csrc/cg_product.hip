@@ -957,14 +957,17 @@ constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1
                                     // slot-2 gradient) slot 2 on the matrix cores
 constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
 
-template <int NK>
+// NK = reduction steps of four rows, NT = 16-column tiles of the m2 axis (1 or 2).  The loop body has
+// no branch: a tile the window of valid m2 does not reach gets zero coefficients.  (With branches
+// around the tiles the compiler copied the accumulators at every join, and each copy waits for
+// the matrix pipeline to drain.)
+template <int NK, int NT>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
                                             int split, int lane, f32x4 (&dre)[2], f32x4 (&dim)[2]) {
     const int l = q.l, l1 = q.l1, l2 = q.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = q.rows, tau2 = q.tau2;
-    const int ntiles = (M2 + 15) >> 4;
     const int i = lane & 15, kk = lane >> 4;
     const int io = min(i, tau2 - 1);                              // rows past the last channel repeat it (never stored)
     // per reduction step: the lane's row of the unit, its tile entry and fragment row
@@ -980,14 +983,12 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
     }
     for (int mi = part; mi < M; mi += split) {
         const int m = mi - l;
-        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);    // valid m2
-        if (hi < lo) continue;
+        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);    // valid m2; never empty since |m| <= l <= l1 + l2
         float2 gq[NK];
 #pragma unroll
         for (int c = 0; c < NK; ++c) gq[c] = g[goff[c] + mi];
 #pragma unroll
-        for (int tile = 0; tile < 2; ++tile) {
-            if (tile >= ntiles || hi + l2 < 16 * tile || lo + l2 > 16 * tile + 15) continue;    // wave-uniform
+        for (int tile = 0; tile < NT; ++tile) {
             const int m2 = 16 * tile + i - l2;                    // this lane's column
             const bool cval = m2 >= lo && m2 <= hi;
             const int m2c = min(max(m2, lo), hi);
@@ -1039,12 +1040,19 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         const float2 *g, *f2;
         bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+#define CGNET_MM(NK_)                                                                       \
+    case NK_:                                                                               \
+        if (cur.l2 <= 7) bwd_mm_task<NK_, 1>(q, cgp, g, c.f1, part, split, lane, dre, dim); \
+        else bwd_mm_task<NK_, 2>(q, cgp, g, c.f1, part, split, lane, dre, dim);             \
+        break;
         switch ((u.rows + 3) >> 2) {
-            case 1: bwd_mm_task<1>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
-            case 2: bwd_mm_task<2>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
-            case 3: bwd_mm_task<3>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
-            default: bwd_mm_task<4>(q, cgp, g, c.f1, part, split, lane, dre, dim); break;
+            CGNET_MM(1) CGNET_MM(2) CGNET_MM(3)
+            default:
+                if (cur.l2 <= 7) bwd_mm_task<4, 1>(q, cgp, g, c.f1, part, split, lane, dre, dim);
+                else bwd_mm_task<4, 2>(q, cgp, g, c.f1, part, split, lane, dre, dim);
+                break;
         }
+#undef CGNET_MM
         if (cur.last_of_l2) {
             const int M2 = 2 * cur.l2 + 1;
             mfma_drain();
