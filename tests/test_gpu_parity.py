@@ -154,6 +154,22 @@ def test_cg_random_shapes(dev, lmax, taus, bsz, mode):
     test_cg_forward_backward(dev, lmax, taus, bsz, mode)
 
 
+def _random_matrix_core_cases(n, seed):
+    """Shapes whose backward takes the kernel with one gradient on the matrix cores: every channel count in 8..16."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        lmax = int(rng.integers(0, 7))
+        taus = [int(rng.integers(8, 17)) for _ in range(lmax + 1)]
+        cases.append((lmax, taus, int(rng.integers(1, 6)), str(rng.choice(["default", "mst", "debug"]))))
+    return cases
+
+
+@pytest.mark.parametrize("lmax,taus,bsz,mode", _random_matrix_core_cases(12, 5))
+def test_cg_random_shapes_matrix_core_backward(dev, lmax, taus, bsz, mode):
+    test_cg_forward_backward(dev, lmax, taus, bsz, mode)
+
+
 @pytest.mark.parametrize("lmax,taus,bsz,mode", [CG_CASES[2], CG_CASES[5], CG_CASES[7]])
 def test_cg_backward_general_kernel(dev, monkeypatch, lmax, taus, bsz, mode):
     """The LDS-accumulator backward kernel (fallback for shapes the register-resident scheme cannot
