@@ -1560,14 +1560,13 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 const int M1 = 2 * u.l1 + 1, tau1 = h_t_F[u.l1];
                 const int r0 = (u.offF1 - p->cumF[u.l1]) / M1;
                 if (u.l1 != cur_l1) { cur_l1 = u.l1; slab_of_piece.clear(); }
-                double acc = 0, piece_cost = 0;
+                double piece_cost = 0;
                 int start = u.task_begin, piece = 0;
                 // all row ranges of a degree have the same task list and costs, hence the same cuts
                 for (int k = u.task_begin; k < u.task_end; ++k) {
-                    acc += task_cost[k];
                     piece_cost += task_cost[k];
                     const bool last = k + 1 == u.task_end;
-                    if (last || (p->bwd_utasks[k].last_of_l2 && acc >= target)) {
+                    if (last || (p->bwd_utasks[k].last_of_l2 && piece_cost >= target)) {
                         BwdUnit v = u;
                         v.task_begin = start;
                         v.task_end = k + 1;
@@ -1582,7 +1581,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                         cut.push_back(v);
                         unit_cost.push_back(piece_cost);
                         start = k + 1;
-                        acc = piece_cost = 0;
+                        piece_cost = 0;
                         ++piece;
                     }
                 }
