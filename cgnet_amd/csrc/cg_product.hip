@@ -1289,9 +1289,21 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 t.offFF = p->cumFF[l] + (p->t_off[i] + r0 * tau2) * M;
                 t.cg_off = cgo[i];
                 t.chan0 = p->cumT[l] + p->t_off[i] + r0 * tau2;
-                t.nT1 = (t.rows + 3) / 4;
+                // Register tile of the forward kernel: the one whose items (tiles x m) fill the waves they
+                // occupy best, weighed by the instructions of one term of the inner loop
+                // (4 TI TJ multiply-adds + 2 TI coefficient products + TI + TJ + 3 address / loop steps).
+                double best_cost = -1;
+                for (int ti = 1; ti <= std::min(4, t.rows); ++ti)
+                    for (int tj = 1; tj <= std::min(4, tau2); ++tj) {
+                        const int n1 = (t.rows + ti - 1) / ti, n2 = (tau2 + tj - 1) / tj;
+                        const long long items = (long long)n1 * n2 * M;
+                        const double cost = (double)((items + 63) / 64) * (4 * ti * tj + 3 * ti + tj + 3);
+                        if (best_cost < 0 || cost < best_cost * (1 - 1e-9)) {
+                            best_cost = cost;
+                            t.nT1 = n1; t.nT2 = n2;
+                        }
+                    }
                 t.TI = (t.rows + t.nT1 - 1) / t.nT1;
-                t.nT2 = (tau2 + 3) / 4;
                 t.TJ = (tau2 + t.nT2 - 1) / t.nT2;
                 t.bTI[0] = t.bTI[1] = 1;
                 t.bRW[0] = t.bRW[1] = 1;
