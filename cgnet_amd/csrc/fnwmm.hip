@@ -187,43 +187,6 @@ pack_w_backward_kernel(const float2* __restrict__ W, const float* __restrict__ s
 }
 
 // --------------------------------------------------------------------------- forward (MFMA)
-// Streaming helper: a contiguous run of n complex numbers starting at element `off` of a
-// (16-byte aligned) float2 array is fetched with 16-byte loads, lane-contiguous, from the
-// element pair that contains `off`; the LDS image therefore starts `off & 1` elements early.
-template <int NREG>
-struct Run16 {
-    float4 r[NREG];
-    // issue the loads (whole work-group, tid = 0..nthreads-1); elements beyond `total` are not touched
-    __device__ __forceinline__ void fetch(const float2* __restrict__ base, size_t off, int n, size_t total, int tid,
-                                          int nthreads) {
-        const size_t first = off & ~(size_t)1;
-        const int n4 = (n + (int)(off & 1) + 1) >> 1;
-        const float4* src = reinterpret_cast<const float4*>(base + first);
-#pragma unroll
-        for (int k = 0; k < NREG; ++k) {
-            const int idx = tid + k * nthreads;
-            r[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (idx < n4) {
-                if (first + 2 * (size_t)idx + 1 < total) {
-                    r[k] = src[idx];
-                } else {
-                    const float2 z = base[first + 2 * (size_t)idx];
-                    r[k] = make_float4(z.x, z.y, 0.f, 0.f);
-                }
-            }
-        }
-    }
-    __device__ __forceinline__ void commit(float2* __restrict__ lds, size_t off, int n, int tid, int nthreads) const {
-        const int n4 = (n + (int)(off & 1) + 1) >> 1;
-        float4* dst = reinterpret_cast<float4*>(lds);
-#pragma unroll
-        for (int k = 0; k < NREG; ++k) {
-            const int idx = tid + k * nthreads;
-            if (idx < n4) dst[idx] = r[k];
-        }
-    }
-};
-
 // s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate); n above the table waits for all.
 __device__ __forceinline__ void wait_vmcnt(int n) {
 #define CGNET_VMCNT(N) case N: __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14)); break;
@@ -422,15 +385,12 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
 }
 
 // --------------------------------------------------------------------------- grad W (MFMA)
-// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples
-// into part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
-constexpr int kGwFFRegs = 4;    // 4 x 256 x 16 B = 16 KB of FF per sample and work-group
-constexpr int kGwGORegs = 3;    // 3 x 256 x 16 B = 12 KB of gO rows (16 rows of up to 95 complex)
-
-// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples
-// into part[chunk][nW].  Per sample the group's FF rows (nc channels x M, one contiguous run) and
-// the 16 gO rows are streamed through LDS with 16-byte lane-contiguous loads, double buffered;
-// each wave then reads its 16 channel rows in matrix-core operand order.
+// Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples into
+// part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
+// Per sample the group's FF rows (nc channels x M, one contiguous run) and the 16 gO rows are copied
+// straight into LDS (LDS-direct loads, no registers), one sample ahead into the other half of a
+// double buffer, one barrier per sample; each wave then reads its 16 channel rows in matrix-core
+// operand order.
 __global__ void __launch_bounds__(kThreads)
 wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, float2* __restrict__ part,
                  const WmmDeg* __restrict__ degs, const WmmChanUnit* __restrict__ units, int B,
@@ -452,34 +412,32 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
     const int go_rows = min(16, d.tO - u.rc * 16);
     const int nblk = (M + 7) >> 3;
     const int n_ff = u.nc * M, n_go = go_rows * M;
-    const size_t tot_ff = (size_t)B * nFF, tot_go = (size_t)B * nO;
     const int b_begin = up.part * samples_per_chunk;
     const int b_end = min(B, b_begin + samples_per_chunk);
 
-    Run16<kGwFFRegs> pf;
-    Run16<kGwGORegs> pg;
-    auto ff_off = [&](int b) { return (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M; };
-    auto go_off = [&](int b) { return (size_t)b * nO + d.cumO + (size_t)u.rc * 16 * M; };
-    if (b_begin < b_end) {
-        pf.fetch(FF, ff_off(b_begin), n_ff, tot_ff, tid, kThreads);
-        pg.fetch(gO, go_off(b_begin), n_go, tot_go, tid, kThreads);
-    }
+    // one sample's FF rows of the unit (one contiguous run) and its gO rows, copied straight into LDS
+    auto issue = [&](int b, int par) {
+        const float2* fsrc = FF + (size_t)b * nFF + d.cumFF + (size_t)u.c0 * M;
+        const float2* gsrc = gO + (size_t)b * nO + d.cumO + (size_t)u.rc * 16 * M;
+        float2* fdst = ffbuf + par * ff_cap;
+        float2* gdst = gobuf + par * go_cap;
+        dma16<kThreads>(fsrc, fdst, n_ff >> 1, tid);
+        if (n_ff & 1) dma8(fsrc + (n_ff - 1), fdst + (n_ff - 1), tid);
+        dma16<kThreads>(gsrc, gdst, n_go >> 1, tid);
+        if (n_go & 1) dma8(gsrc + (n_go - 1), gdst + (n_go - 1), tid);
+    };
+    if (b_begin < b_end) issue(b_begin, 0);
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
     int buf = 0;
     for (int b = b_begin; b < b_end; ++b, buf ^= 1) {
-        float2* ffl = ffbuf + buf * ff_cap;
-        float2* gol = gobuf + buf * go_cap;
-        const size_t fo = ff_off(b), go_ = go_off(b);
-        pf.commit(ffl, fo, n_ff, tid, kThreads);
-        pg.commit(gol, go_, n_go, tid, kThreads);
-        __syncthreads();
-        if (b + 1 < b_end) {
-            pf.fetch(FF, ff_off(b + 1), n_ff, tot_ff, tid, kThreads);
-            pg.fetch(gO, go_off(b + 1), n_go, tot_go, tid, kThreads);
-        }
+        const float2* ffl = ffbuf + buf * ff_cap;
+        const float2* gol = gobuf + buf * go_cap;
+        dma_wait();
+        __syncthreads();           // sample b landed; nobody still reads the other buffer
+        if (b + 1 < b_end) issue(b + 1, buf ^ 1);
         if (wave_on) {
-            const float2* frow = ffl + (fo & 1) + (cok ? (16 * w + i) : 0) * M;
-            const float2* grow = gol + (go_ & 1) + (tok ? i : 0) * M;
+            const float2* frow = ffl + (cok ? (16 * w + i) : 0) * M;
+            const float2* grow = gol + (tok ? i : 0) * M;
             for (int blk = 0; blk < nblk; ++blk) {
                 const int p0 = blk * 8 + kk * 2;
                 float2 f0 = make_float2(0.f, 0.f), f1 = f0, g0 = f0, g1 = f0;
@@ -864,7 +822,8 @@ extern "C" int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_
                 p->fwd_units.push_back(u);
             }
         int gw_nc = 64;
-        while (gw_nc > 16 && (size_t)gw_nc * d.M + 2 > (size_t)kGwFFRegs * kThreads * 2) gw_nc /= 2;
+        // both stages of the unit's FF rows and of the 16 gO rows fit 64 KB of LDS
+        while (gw_nc > 16 && 16 * ((size_t)gw_nc * d.M + 2 + 16 * (size_t)d.M + 2) > 64 * 1024) gw_nc /= 2;
         for (int rc = 0; rc < d.nrc; ++rc)
             for (int c0 = 0; c0 < d.K; c0 += gw_nc)
                 p->gw_units.push_back(WmmChanUnit{di, rc, c0, std::min(gw_nc, d.K - c0)});
