@@ -385,6 +385,39 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
 }
 
 // --------------------------------------------------------------------------- grad W (MFMA)
+// NB blocks of eight m positions of one sample: all operands are read first, then the matrix
+// instructions run back to back.  Positions past the end of the row read the last entry instead
+// and get a zero gO operand; lanes without a channel or an output row read row 0 (their columns /
+// rows of the accumulator are never stored).
+template <int NB>
+__device__ __forceinline__ void gradw_blocks(const float2* __restrict__ frow, const float2* __restrict__ grow,
+                                             int blk0, int M, int kk, bool tok, f32x4& acc0, f32x4& acc1) {
+    float2 f[NB][2], g[NB][2];
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int p = (blk0 + blk) * 8 + kk * 2 + j;
+            const int pc = min(p, M - 1);
+            f[blk][j] = frow[pc];
+            const float2 z = grow[pc];
+            const bool on = tok && p < M;
+            g[blk][j] = make_float2(on ? z.x : 0.f, on ? z.y : 0.f);
+        }
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) {
+        const float2 f0 = f[blk][0], f1 = f[blk][1], g0 = g[blk][0], g1 = g[blk][1];
+        acc0 = mfma4(g0.x, f0.x, acc0);
+        acc0 = mfma4(g0.y, f0.y, acc0);
+        acc0 = mfma4(g1.x, f1.x, acc0);
+        acc0 = mfma4(g1.y, f1.y, acc0);
+        acc1 = mfma4(g0.y, f0.x, acc1);
+        acc1 = mfma4(-g0.x, f0.y, acc1);
+        acc1 = mfma4(g1.y, f1.x, acc1);
+        acc1 = mfma4(-g1.x, f1.y, acc1);
+    }
+}
+
 // Raw sums  sum_{b in chunk, m} gO[b,to,m] * conj(FF[b,c,m])  of one chunk of samples into
 // part[chunk][nW]; wmm_gradw_finish_kernel adds the chunks in order and divides by div[c].
 // Per sample the group's FF rows (nc channels x M, one contiguous run) and the 16 gO rows are copied
@@ -438,25 +471,18 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
         if (wave_on) {
             const float2* frow = ffl + (cok ? (16 * w + i) : 0) * M;
             const float2* grow = gol + (tok ? i : 0) * M;
-            for (int blk = 0; blk < nblk; ++blk) {
-                const int p0 = blk * 8 + kk * 2;
-                float2 f0 = make_float2(0.f, 0.f), f1 = f0, g0 = f0, g1 = f0;
-                if (p0 < M) {
-                    if (cok) f0 = frow[p0];
-                    if (tok) g0 = grow[p0];
-                }
-                if (p0 + 1 < M) {
-                    if (cok) f1 = frow[p0 + 1];
-                    if (tok) g1 = grow[p0 + 1];
-                }
-                acc0 = mfma4(g0.x, f0.x, acc0);
-                acc0 = mfma4(g0.y, f0.y, acc0);
-                acc0 = mfma4(g1.x, f1.x, acc0);
-                acc0 = mfma4(g1.y, f1.y, acc0);
-                acc1 = mfma4(g0.y, f0.x, acc1);
-                acc1 = mfma4(-g0.x, f0.y, acc1);
-                acc1 = mfma4(g1.y, f1.x, acc1);
-                acc1 = mfma4(-g1.x, f1.y, acc1);
+            switch (nblk) {
+                case 1: gradw_blocks<1>(frow, grow, 0, M, kk, tok, acc0, acc1); break;
+                case 2: gradw_blocks<2>(frow, grow, 0, M, kk, tok, acc0, acc1); break;
+                case 3: gradw_blocks<3>(frow, grow, 0, M, kk, tok, acc0, acc1); break;
+                case 4: gradw_blocks<4>(frow, grow, 0, M, kk, tok, acc0, acc1); break;
+                default:
+                    for (int blk = 0; blk < nblk; blk += 3) {
+                        if (blk + 3 <= nblk) gradw_blocks<3>(frow, grow, blk, M, kk, tok, acc0, acc1);
+                        else if (blk + 2 == nblk) gradw_blocks<2>(frow, grow, blk, M, kk, tok, acc0, acc1);
+                        else gradw_blocks<1>(frow, grow, blk, M, kk, tok, acc0, acc1);
+                    }
+                    break;
             }
         }
     }
