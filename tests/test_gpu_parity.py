@@ -437,6 +437,28 @@ def test_layer_random_shapes(dev, lmax, tin, tout, bsz, sparse, bn, k):
         assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W")
 
 
+def test_layer_backward_two_streams_matches_one_stream(dev, monkeypatch):
+    """The layer's backward runs the weight gradient on a second stream; several steps back to back, without a
+    host synchronisation in between, must give bit for bit what the same steps give on one stream."""
+    from cgnet_amd import CG_layers
+    lmax, tin, tout, bsz = 6, [9, 8, 12, 10, 16, 8, 11], [8] * 7, 7
+    x = rand_straight(tin, bsz, seed=31).float().to(dev)
+    g = torch.Generator().manual_seed(33)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    gos = [torch.randn(bsz, n_o, 2, generator=g).to(dev) for _ in range(4)]
+    results = []
+    for overlap in (1, 0):
+        monkeypatch.setattr(CG_layers, "_OVERLAP_GRAD_W", overlap)
+        mod, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=7)
+        mod.train()
+        xs = x.clone().requires_grad_(True)
+        for go in gos:                                   # gradients accumulate over the steps
+            mod(xs, straight_output=True).backward(go)
+        results.append((xs.grad.clone(), mod.bnWMM.W.grad.clone(), mod.bnWMM.bn_stds.detach().clone()))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
 def test_spherical_cnn_stack(dev):
     from cgnet_amd import CGNet
     lmax = 4
