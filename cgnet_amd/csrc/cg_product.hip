@@ -1156,6 +1156,7 @@ cg_backward_combine_kernel(const float2* __restrict__ part1, const float2* __res
     float2 s = make_float2(0.f, 0.f);
     if (own1[lam]) s = part1[idx];
     const float2* p2 = part2 + (size_t)b * P2;
+#pragma unroll 8
     for (int k = lbeg[lam]; k < lbeg[lam + 1]; ++k) {
         const float2 v = p2[loff[k] + rel];
         s.x += v.x;
