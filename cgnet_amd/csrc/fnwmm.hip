@@ -376,6 +376,7 @@ wmm_sum_slices_kernel(const float2* __restrict__ part, float2* __restrict__ O,
     if (idx >= (size_t)B * nO) return;
     const int S = cumO_S[ndeg + 1 + di];
     float2 s = part[idx];
+#pragma unroll 8
     for (int k = 1; k < S; ++k) {
         const float2 v = part[(size_t)k * B * nO + idx];
         s.x += v.x;
