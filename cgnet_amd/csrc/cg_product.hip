@@ -960,7 +960,10 @@ constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
 // NK = reduction steps of four rows, NT = 16-column tiles of the m2 axis (1 or 2).  The loop body has
 // no branch: a tile the window of valid m2 does not reach gets zero coefficients.  (With branches
 // around the tiles the compiler copied the accumulators at every join, and each copy waits for
-// the matrix pipeline to drain.)
+// the matrix pipeline to drain.)  All addresses are explicit LDS byte addresses advanced by
+// constants from one m to the next.  The table holds zeros where m - m2 is no valid m1 (every
+// table this library fills does), so only the columns past the end of the m2 axis are masked;
+// the fragment column of such an entry is clamped into its row and multiplied by that zero.
 template <int NK, int NT>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
@@ -970,42 +973,65 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
     const int rows = q.rows, tau2 = q.tau2;
     const int i = lane & 15, kk = lane >> 4;
     const int io = min(i, tau2 - 1);                              // rows past the last channel repeat it (never stored)
-    // per reduction step: the lane's row of the unit, its tile entry and fragment row
-    int goff[NK], foff[NK];
-    bool kval[NK];
+    // per reduction step: LDS address of the lane's tile entry at m index `part`, base of its fragment row;
+    // rows past the end of the unit repeat the last one and get a zero coefficient
+    unsigned ga[NK], fbase[NK];
+    float kmask[NK];
 #pragma unroll
     for (int c = 0; c < NK; ++c) {
         const int k = 4 * c + kk;
         const int kc = min(k, rows - 1);
-        kval[c] = k < rows;
-        goff[c] = (kc * tau2 + io) * M;
-        foff[c] = kc * (M1 + 1);
+        kmask[c] = k < rows ? 1.f : 0.f;
+        ga[c] = opaque(lds_addr(g + (kc * tau2 + io) * M + part));
+        fbase[c] = lds_addr(f1 + kc * (M1 + 1));
     }
+    const bool kfull = (rows & 3) == 0;                           // uniform: no step needs the mask
+    // per tile: address of the lane's coefficient at m index `part`, whether its column exists, and
+    // fragment column minus m index (column of slot 1 = m - m2 + l1)
+    unsigned ca[NT];
+    bool colok[NT];
+    int fc0[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int col = 16 * t + i;
+        const int colc = min(col, M2 - 1);
+        colok[t] = col < M2;
+        ca[t] = opaque(lds_addr(cgp + (kTabLo + part) * M2 + colc));
+        fc0[t] = part - l - (colc - l2) + l1;
+    }
+    const unsigned gstep = 8u * (unsigned)split, cstep = 4u * (unsigned)(split * M2);
     for (int mi = part; mi < M; mi += split) {
-        const int m = mi - l;
-        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);    // valid m2; never empty since |m| <= l <= l1 + l2
         float2 gq[NK];
+        float ngy[NK];
 #pragma unroll
-        for (int c = 0; c < NK; ++c) gq[c] = g[goff[c] + mi];
+        for (int c = 0; c < NK; ++c) {
+            gq[c] = lds_c(ga[c], 0);
+            ga[c] += gstep;
+        }
+        float cc[NT];
+        float2 fq[NT][NK];
 #pragma unroll
-        for (int tile = 0; tile < NT; ++tile) {
-            const int m2 = 16 * tile + i - l2;                    // this lane's column
-            const bool cval = m2 >= lo && m2 <= hi;
-            const int m2c = min(max(m2, lo), hi);
-            const float cc = cgp[(kTabLo + mi) * M2 + m2c + l2];
-            const float cv = cval ? cc : 0.f;
-            const int fcol = m - m2c + l1;                        // column of the slot-1 fragment
-            float2 fq[NK];
+        for (int t = 0; t < NT; ++t) {
+            cc[t] = lds_f(ca[t])[0];
+            ca[t] += cstep;
+            const int fcol = max(0, min(M1 - 1, fc0[t]));         // clamped where the coefficient is zero anyway
+            fc0[t] += split;
 #pragma unroll
-            for (int c = 0; c < NK; ++c) fq[c] = f1[foff[c] + fcol];
+            for (int c = 0; c < NK; ++c) fq[t][c] = lds_c(fbase[c] + 8u * (unsigned)fcol, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < NK; ++c) ngy[c] = -gq[c].y;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float cv = colok[t] ? cc[t] : 0.f;
 #pragma unroll
             for (int c = 0; c < NK; ++c) {
-                const float w = kval[c] ? cv : 0.f;
-                const float bx = w * fq[c].x, by = -w * fq[c].y;  // C conj(f)
-                dre[tile] = mfma4(gq[c].x, bx, dre[tile]);
-                dim[tile] = mfma4(gq[c].x, by, dim[tile]);
-                dre[tile] = mfma4(-gq[c].y, by, dre[tile]);
-                dim[tile] = mfma4(gq[c].y, bx, dim[tile]);
+                const float w = kfull ? cv : cv * kmask[c];
+                const float bx = w * fq[t][c].x, by = -w * fq[t][c].y;  // C conj(f)
+                dre[t] = mfma4(gq[c].x, bx, dre[t]);
+                dim[t] = mfma4(gq[c].x, by, dim[t]);
+                dre[t] = mfma4(ngy[c], by, dre[t]);
+                dim[t] = mfma4(gq[c].y, bx, dim[t]);
             }
         }
     }
