@@ -964,7 +964,7 @@ constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
 // constants from one m to the next.  The table holds zeros where m - m2 is no valid m1 (every
 // table this library fills does), so only the columns past the end of the m2 axis are masked;
 // the fragment column of such an entry is clamped into its row and multiplied by that zero.
-template <int NK, int NT>
+template <int NK, int NT, bool KFULL>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
                                             int split, int lane, f32x4 (&dre)[2], f32x4 (&dim)[2]) {
@@ -985,7 +985,6 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
         ga[c] = opaque(lds_addr(g + (kc * tau2 + io) * M + part));
         fbase[c] = lds_addr(f1 + kc * (M1 + 1));
     }
-    const bool kfull = (rows & 3) == 0;                           // uniform: no step needs the mask
     // per tile: address of the lane's coefficient at m index `part`, whether its column exists, and
     // fragment column minus m index (column of slot 1 = m - m2 + l1)
     unsigned ca[NT];
@@ -1023,10 +1022,10 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
         for (int c = 0; c < NK; ++c) ngy[c] = -gq[c].y;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const float cv = colok[t] ? cc[t] : 0.f;
+            const float cv = (NT == 2 && t == 0) || colok[t] ? cc[t] : 0.f;   // two tiles: the first one is full
 #pragma unroll
             for (int c = 0; c < NK; ++c) {
-                const float w = kfull ? cv : cv * kmask[c];
+                const float w = KFULL ? cv : cv * kmask[c];   // KFULL: the rows fill every step of four
                 const float bx = w * fq[t][c].x, by = -w * fq[t][c].y;  // C conj(f)
                 dre[t] = mfma4(gq[c].x, bx, dre[t]);
                 dim[t] = mfma4(gq[c].x, by, dim[t]);
@@ -1066,18 +1065,30 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         const float2 *g, *f2;
         bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
-#define CGNET_MM(NK_)                                                                       \
-    case NK_:                                                                               \
-        if (cur.l2 <= 7) bwd_mm_task<NK_, 1>(q, cgp, g, c.f1, part, split, lane, dre, dim); \
-        else bwd_mm_task<NK_, 2>(q, cgp, g, c.f1, part, split, lane, dre, dim);             \
+#define CGNET_MM_CALL(NK_, NT_, KF_) bwd_mm_task<NK_, NT_, KF_>(q, cgp, g, c.f1, part, split, lane, dre, dim)
+#define CGNET_MM(NK_)                                                   \
+    case NK_:                                                           \
+        if (cur.l2 <= 7) {                                              \
+            if (u.rows & 3) CGNET_MM_CALL(NK_, 1, false);               \
+            else CGNET_MM_CALL(NK_, 1, true);                           \
+        } else {                                                        \
+            if (u.rows & 3) CGNET_MM_CALL(NK_, 2, false);               \
+            else CGNET_MM_CALL(NK_, 2, true);                           \
+        }                                                               \
         break;
         switch ((u.rows + 3) >> 2) {
             CGNET_MM(1) CGNET_MM(2) CGNET_MM(3)
             default:
-                if (cur.l2 <= 7) bwd_mm_task<4, 1>(q, cgp, g, c.f1, part, split, lane, dre, dim);
-                else bwd_mm_task<4, 2>(q, cgp, g, c.f1, part, split, lane, dre, dim);
+                if (cur.l2 <= 7) {
+                    if (u.rows & 3) CGNET_MM_CALL(4, 1, false);
+                    else CGNET_MM_CALL(4, 1, true);
+                } else {
+                    if (u.rows & 3) CGNET_MM_CALL(4, 2, false);
+                    else CGNET_MM_CALL(4, 2, true);
+                }
                 break;
         }
+#undef CGNET_MM_CALL
 #undef CGNET_MM
         if (cur.last_of_l2) {
             const int M2 = 2 * cur.l2 + 1;
