@@ -1506,7 +1506,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                             // a matrix instruction occupies its pipeline for eight vector-instruction slots
                             const int Mq = 2 * tl[tri[k]] + 1;
                             const int split = kHybWaves - nA;
-                            bc = ((Mq + split - 1) / split) * (double)((M2 + 15) / 16) * (((rows_c + 3) / 4) * 32.0 + 26.0);
+                            bc = ((Mq + split - 1) / split) * (double)((M2 + 15) / 16) * (((rows_c + 3) / 4) * 32.0 + 18.0);
                             bTI[k] = 1; bRW[k] = 1;
                         }
                         for (int ti = 1; ti <= kBwdMaxTI && !hybrid; ++ti)
