@@ -1219,7 +1219,7 @@ partial_sum_kernel(const float2* __restrict__ part, float2* __restrict__ out, si
 int samples_per_group_for(int B, int ntasks) {
     // enough work-groups to fill 256 CUs a few times over, while each group amortises the
     // staging of its CG table over several samples
-    int groups = std::max(1, std::min(B, (4096 + ntasks - 1) / std::max(1, ntasks)));
+    int groups = std::max(1, std::min(B, (6144 + ntasks - 1) / std::max(1, ntasks)));
     return (B + groups - 1) / groups;
 }
 
