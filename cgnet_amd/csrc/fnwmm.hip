@@ -142,31 +142,40 @@ fn_update_std_kernel(const double* __restrict__ sums, float* __restrict__ stds,
 }
 
 // --------------------------------------------------------------------------- weight packing
-// Forward operand: for every degree, k-step ks (4 channels), row chunk rc: two 64-lane blocks
-// (rows = W_re, rows = W_im), lane 16*kk + row holds W[rc*16+row][4*ks+kk] / div.
+// Forward operand: for every degree, block of 8 channels kb and row chunk rc: 256 floats, lane-major,
+// four per lane = (k-step 0 | 1) x (W_re | W_im) of W[rc*16+row][kb*8 + 4*step + kk] / div with
+// lane = 16*kk + row.  One thread writes the four floats of one lane (two weights, one 16-byte store).
 __global__ void __launch_bounds__(256)
 pack_w_forward_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                       const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int total_blocks) {
     __shared__ int s_tab[kMaxLookup];
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int blk = idx >> 6;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // one per (group of 256 floats, lane)
+    const int blk = idx >> 4;                                     // 64-float block of the packed array
     const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].wp_base; }, s_tab);
     if (blk >= total_blocks) return;
     const WmmDeg d = degs[di];
-    // 256 floats per (block of 8 channels, row chunk): lane-major, 4 per lane = (step, re/im rows)
-    const int rel = idx - d.wp_base * 64;
-    const int sub = rel & 3, lane = (rel >> 2) & 63, grp = rel >> 8;
-    const int tile = sub & 1, step = sub >> 1;
+    const int rel = idx - d.wp_base * 16;
+    const int lane = rel & 63, grp = rel >> 6;
     const int rc = grp % d.nrc, kb = grp / d.nrc;
     const int row = lane & 15, kk = lane >> 4;
-    const int to = rc * 16 + row, c = kb * 8 + step * 4 + kk;
-    float v = 0.f;
-    if (to < d.tO && c < d.K) {
-        const float2 w = W[d.cumW + (size_t)to * d.K + c];
-        v = tile ? w.y : w.x;
-        if (stds) v /= fmaxf(eps, stds[d.cumT + c]);
+    const int to = rc * 16 + row;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (to < d.tO) {
+        const int c0 = kb * 8 + kk, c1 = c0 + 4;
+        const float2* wrow = W + d.cumW + (size_t)to * d.K;
+        float2 w0 = make_float2(0.f, 0.f), w1 = w0;
+        float r0 = 1.f, r1 = 1.f;
+        if (c0 < d.K) {
+            w0 = wrow[c0];
+            if (stds) r0 = fmaxf(eps, stds[d.cumT + c0]);
+        }
+        if (c1 < d.K) {
+            w1 = wrow[c1];
+            if (stds) r1 = fmaxf(eps, stds[d.cumT + c1]);
+        }
+        v = stds ? make_float4(w0.x / r0, w0.y / r0, w1.x / r1, w1.y / r1) : make_float4(w0.x, w0.y, w1.x, w1.y);
     }
-    Wp[idx] = v;
+    reinterpret_cast<float4*>(Wp)[idx] = v;
 }
 
 // Backward operand: WT[cumW + c*tO + to] = conj(W[to][c]) / div[c]
@@ -564,23 +573,26 @@ __global__ void __launch_bounds__(256)
 pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                      const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Ap, int total_blocks) {
     __shared__ int s_tab[kMaxLookup];
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int blk = idx >> 6, lane = idx & 63;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // one weight = two packed floats
+    const int blk = idx >> 5, half = (idx >> 4) & 1, i = idx & 15;
     const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].ap_base; }, s_tab);
     if (blk >= total_blocks) return;
     const WmmDeg d = degs[di];
     const int rel = blk - d.ap_base;             // ctile * nks_b + ks
     const int ks = rel % d.nks_b, ctile = rel / d.nks_b;
-    const int i = lane & 15, kk = lane >> 4;
-    const int c = ctile * 16 + i, k = 4 * ks + kk;
-    const int to = k >> 1, sel = k & 1;
-    float v = 0.f;
+    const int c = ctile * 16 + i, to = 2 * ks + half;             // k = 4*ks + kk, to = k >> 1, kk = 2*half + sel
+    float2 w = make_float2(0.f, 0.f);
     if (c < d.K && to < d.tO) {
-        const float2 w = W[d.cumW + (size_t)to * d.K + c];
-        v = sel ? w.y : w.x;
-        if (stds) v /= fmaxf(eps, stds[d.cumT + c]);
+        w = W[d.cumW + (size_t)to * d.K + c];
+        if (stds) {
+            const float r = fmaxf(eps, stds[d.cumT + c]);
+            w.x /= r;
+            w.y /= r;
+        }
     }
-    Ap[idx] = v;
+    float* dst = Ap + (size_t)blk * 64 + half * 32 + i;
+    dst[0] = w.x;
+    dst[16] = w.y;
 }
 
 // Gradient with respect to FF on the matrix cores (t_O <= 16): gFF[c, (m, re/im)] = sum_k A[c, k] * B[k, (m, re/im)]
@@ -990,7 +1002,7 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
         return CGNET_OK;
     }
     float* Wp = (float*)(base + ws.wp);
-    const int total = plan->wp_blocks * 64;
+    const int total = plan->wp_blocks * 16;   // one thread per four packed floats
     CGNET_LAUNCH(pack_w_forward_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
                        bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Wp, plan->wp_blocks);
     CGNET_HIP(hipGetLastError());
@@ -1089,7 +1101,7 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
         if (plan->gff_mfma && plan->nW > 0 && plan->nO > 0) {
             float* Ap = (float*)d_workspace;
-            const int total = plan->ap_blocks * 64;
+            const int total = plan->ap_blocks * 32;   // one thread per weight
             CGNET_LAUNCH(pack_w_gradff_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
                          bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Ap, plan->ap_blocks);
             CGNET_HIP(hipGetLastError());
