@@ -32,6 +32,7 @@ struct Pending { const char* name; hipEvent_t start, stop; };
 struct Total { double ms = 0.; int launches = 0; };
 std::mutex g_mu;
 bool g_enabled = false;
+std::string g_only;              // when set, only launches of this kernel are timed
 std::vector<Pending> g_pending;
 std::vector<hipEvent_t> g_pool;
 std::map<std::string, Total> g_totals;
@@ -51,6 +52,7 @@ hipEvent_t take_event() {
 KernelTimer::KernelTimer(const char* name, hipStream_t stream) : name_(name), stream_(stream) {
     std::lock_guard<std::mutex> lock(g_mu);
     if (!g_enabled) return;
+    if (!g_only.empty() && std::strncmp(name, g_only.c_str(), g_only.size()) != 0) return;
     start_ = take_event();
     stop_ = take_event();
     if (start_ && stop_) {
@@ -75,6 +77,12 @@ extern "C" int cgnet_profile_enable(int on) {
     const int prev = cgnet::g_enabled ? 1 : 0;
     cgnet::g_enabled = on != 0;
     return prev;
+}
+
+extern "C" int cgnet_profile_select(const char* kernel_name) {
+    std::lock_guard<std::mutex> lock(cgnet::g_mu);
+    cgnet::g_only = kernel_name ? kernel_name : "";
+    return CGNET_OK;
 }
 
 extern "C" int cgnet_profile_reset(void) {

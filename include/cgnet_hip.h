@@ -144,8 +144,12 @@ int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* 
  * recorded on the launch stream.  After the caller has synchronised those streams,
  * cgnet_profile_collect() folds the finished pairs into per-kernel totals and returns the
  * number of distinct kernels; cgnet_profile_get(i, ...) reads entry i (name, summed
- * milliseconds, launches).  cgnet_profile_enable returns the previous setting. */
+ * milliseconds, launches).  cgnet_profile_enable returns the previous setting.
+ * cgnet_profile_select("kernel") restricts the bracketing to launches of that one kernel
+ * (recording events costs a few microseconds per launch, which a timed region that only wants
+ * one kernel's duration need not pay for the others); NULL or "" selects every kernel again. */
 int cgnet_profile_enable(int on);
+int cgnet_profile_select(const char* kernel_name);
 int cgnet_profile_reset(void);
 int cgnet_profile_collect(void);
 int cgnet_profile_get(int index, char* name, int name_capacity, double* total_ms, int* launches);
