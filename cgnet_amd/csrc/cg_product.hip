@@ -134,13 +134,9 @@ __device__ __forceinline__ unsigned opaque(unsigned v) {
 
 
 // ------------------------------------------------------------------------------------ forward
-// Square root from the hardware reciprocal square root plus one Newton step (error below one
-// ulp); sqrt_refined(0) = 0.
-__device__ __forceinline__ float sqrt_refined(float n) {
-    const float y = __builtin_amdgcn_rsqf(fmaxf(n, 1e-37f));
-    const float s = n * y;
-    return fmaf(fmaf(-s, s, n), 0.5f * y, s);
-}
+// The hardware square root (one instruction, error within one ulp).  The statistics use the same
+// rounded modulus in both of their sums, so its last bit does not matter to the variance.
+__device__ __forceinline__ float sqrt_hw(float n) { return __builtin_amdgcn_sqrtf(n); }
 
 // One item = one m of a TI x TJ tile of channels.  Items are ordered m-major, so the lanes of a
 // wave work on a few m with similar numbers of terms, for all channel tiles.  What an item needs
@@ -320,7 +316,7 @@ __device__ __forceinline__ void fwd_group(const CgTask& t, const float2* __restr
                     double a = s1[k], q = s2[k];
                     for (int mm = 0; mm < M; ++mm) {
                         const float2 z = out[ch * M + mm];
-                        const double r = (double)sqrt_refined(fmaf(z.x, z.x, z.y * z.y));
+                        const double r = (double)sqrt_hw(fmaf(z.x, z.x, z.y * z.y));
                         a += r;
                         q = fma(r, r, q);
                     }
