@@ -1331,7 +1331,9 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     for (int tj = 1; tj <= std::min(4, tau2); ++tj) {
                         const int n1 = (t.rows + ti - 1) / ti, n2 = (tau2 + tj - 1) / tj;
                         const long long items = (long long)n1 * n2 * M;
-                        const double cost = (double)((items + 63) / 64) * (4 * ti * tj + 3 * ti + tj + 3);
+                        double cost = (double)((items + 63) / 64) * (4 * ti * tj + 3 * ti + tj + 3);
+                        // more items than threads: the per-item set-up is redone for every sample
+                        if (items > kThreads) cost *= 1.25;
                         if (best_cost < 0 || cost < best_cost * (1 - 1e-9)) {
                             best_cost = cost;
                             t.nT1 = n1; t.nT2 = n2;
