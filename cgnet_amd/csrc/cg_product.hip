@@ -147,7 +147,6 @@ struct FwdItem {
     unsigned pc, pc_end;       // table entries of the first / last term
     int obase;                 // index in the output tile of (first channel of the tile, m)
     int valid;                 // bit i*TJ+j: channel (i, j) of the tile exists
-    bool any;                  // the m has at least one term
 };
 
 template <int TI, int TJ>
@@ -176,8 +175,7 @@ __device__ __forceinline__ void fwd_item_setup(const CgTask& t, int item, const 
 #pragma unroll
     for (int j = 0; j < TJ; ++j) it.pb[j] = lds_addr(f2 + min(tj + nT2 * j, tau2 - 1) * M2 + l2 + lo);
     it.pc = lds_addr(cg + mm * M2 + l2 + lo);
-    it.pc_end = it.pc + 4u * (unsigned)(hi - lo);
-    it.any = hi >= lo;
+    it.pc_end = it.pc + 4u * (unsigned)(hi - lo);   // hi >= lo: the plan only admits triples that obey the triangle rule
     it.obase = (ti * tau2 + tj) * M + mm;
 }
 
@@ -197,9 +195,10 @@ __device__ __forceinline__ void fwd_item_run(const CgTask& t, const FwdItem<TI, 
     for (int j = 0; j < TJ; ++j) pb[j] = opaque(it.pb[j] + bufofs);
     unsigned pc = opaque(it.pc);
     const unsigned pc_end = it.pc_end;
-    if (it.any) {
+    {
+        // every m has at least one term (pc <= pc_end on entry)
 #pragma unroll 2
-        for (; pc <= pc_end; pc += 4u) {
+        do {
             const float c = lds_f(pc)[0];
             float2 b[TJ];
 #pragma unroll
@@ -218,7 +217,8 @@ __device__ __forceinline__ void fwd_item_run(const CgTask& t, const FwdItem<TI, 
                     ai[i][j] = fmaf(a.y, b[j].x, ai[i][j]);
                 }
             }
-        }
+            pc += 4u;
+        } while (pc <= pc_end);
     }
     const int M = 2 * t.l + 1;
     const int si = t.nT1 * t.tau2 * M, sj = t.nT2 * M;
