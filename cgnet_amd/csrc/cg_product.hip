@@ -952,6 +952,10 @@ constexpr int kHybThreads = 512;
 constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
                                     // slot-2 gradient) slot 2 on the matrix cores
 constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
+// Plan: weight of a vector-ALU step of slot 1 against the matrix-core cost of slot 2 in the same
+// work-group.  Measured, not derived: below one because the matrix waves also wait on their operand
+// loads, so a unit is better off with one vector wave fewer than the instruction counts suggest.
+constexpr double kHybSlot1Scale = 0.6;
 
 // NK = reduction steps of four rows, NT = 16-column tiles of the m2 axis (1 or 2).  The loop body has
 // no branch: a tile the window of valid m2 does not reach gets zero coefficients.  (With branches
@@ -1530,7 +1534,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                             std::vector<double> tcost(nt);
                             for (int k = 0; k < nt; ++k) {
                                 const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
-                                const double cA = ((tau2 + rw - 1) / rw) * (double)M2 * (8.0 * ti + 14.0);
+                                const double scaleA = hybrid ? kHybSlot1Scale : 1.0;
+                                const double cA = scaleA * ((tau2 + rw - 1) / rw) * (double)M2 * (8.0 * ti + 14.0);
                                 const double stage = 12.0 * rows_c * tau2 * (2 * tl[tri[k]] + 4) / kThreads + 200.0;
                                 tcost[k] = std::max(cA, costB[k]) + stage;
                                 total += tcost[k];
