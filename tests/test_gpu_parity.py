@@ -712,3 +712,43 @@ def test_errors(dev):
     # empty batch is a no-op
     y = mod(torch.zeros(0, 9, 2, device=dev))
     assert y.shape[0] == 0
+
+
+# ------------------------------------------------------------------------------- timing hooks
+def test_kernel_timing_hooks(dev):
+    """Every launch is bracketed when timing is on; cgnet_profile_select narrows it to one kernel."""
+    from cgnet_amd import CG_layers, _lib
+    lib = _lib.load()
+    mod = CG_layers.CG_woFilter_cuda(3, [2, 2, 2, 2], device=dev)
+    x = rand_straight([2, 2, 2, 2], 3, 1).float().to(dev).requires_grad_(True)
+
+    def step():
+        x.grad = None
+        mod(x, straight_output=True).sum().backward()
+        torch.cuda.synchronize()
+
+    step()
+    try:
+        lib.cgnet_profile_reset()
+        lib.cgnet_profile_select(None)
+        lib.cgnet_profile_enable(1)
+        step()
+        step()
+        lib.cgnet_profile_enable(0)
+        every = _lib.kernel_times()
+        assert "cg_forward_kernel" in every and len(every) >= 2
+        assert every["cg_forward_kernel"][1] == 2 and every["cg_forward_kernel"][0] > 0
+        lib.cgnet_profile_reset()
+        lib.cgnet_profile_select(b"cg_forward_kernel")
+        lib.cgnet_profile_enable(1)
+        step()
+        lib.cgnet_profile_enable(0)
+        only = _lib.kernel_times()
+        assert list(only) == ["cg_forward_kernel"] and only["cg_forward_kernel"][1] == 1
+        lib.cgnet_profile_reset()
+        step()                                            # timing off: nothing recorded
+        assert _lib.kernel_times() == {}
+    finally:
+        lib.cgnet_profile_enable(0)
+        lib.cgnet_profile_select(None)
+        lib.cgnet_profile_reset()
