@@ -98,8 +98,10 @@ template <int NT>
 __device__ __forceinline__ void dma16(const void* __restrict__ src, void* dst, int nchunks, int tid) {
     const char* s = reinterpret_cast<const char*>(src);
     char* d = reinterpret_cast<char*>(dst);
-    for (int e = tid; e < nchunks; e += NT)
-        __builtin_amdgcn_global_load_lds(s + 16 * (size_t)e, (lds_void_ptr)(d + 16 * (e & ~63)), 16, 0, 0);
+    // a 32-bit byte offset from the (wave-uniform) source: one vector add per piece instead of 64-bit address arithmetic
+    const unsigned end = 16u * (unsigned)nchunks;
+    for (unsigned off = 16u * (unsigned)tid; off < end; off += 16u * NT)
+        __builtin_amdgcn_global_load_lds(s + off, (lds_void_ptr)(d + (off & ~1023u)), 16, 0, 0);
 }
 
 // One complex entry (8 bytes, any 8-byte alignment on both sides) copied by lanes 0 and 1 of the
