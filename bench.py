@@ -166,8 +166,8 @@ def main():
     # HBM bytes per launch at this workload from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
     # profiles/cg_layer_L11_tau12_B100_hbm_traffic_pmc.txt (calibrated against a copy kernel of known size)
     measured_traffic = {
-        "cg_backward_hybrid_kernel": 809.9e6, "cg_forward_kernel": 796.1e6, "wmm_forward_kernel": 925.3e6,
-        "wmm_gradw_kernel": 808.4e6, "wmm_gradff_mfma_kernel": 832.5e6,
+        "cg_backward_hybrid_kernel": 809.9e6, "cg_forward_kernel": 796.1e6, "wmm_forward_kernel": 925.2e6,
+        "wmm_gradw_kernel": 807.5e6, "wmm_gradff_mfma_kernel": 832.5e6,
     }
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
     kernels = {}
