@@ -942,7 +942,7 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
 // For a fixed m of the tile, G_m = gFF[t1, t2, m] is a rows x tau2 complex matrix and
 //   gF2[t2, m2] += sum_t1 G_m[t1, t2] * (C[m][m2] conj F1[t1][m - m2])       (tau2 x rows)(rows x window of m2)
 // is a small matrix product: rows of the accumulator = the up to 16 channels of degree l2, columns
-// = up to two tiles of 16 values of m2, reduction over the up to 16 rows of the unit in steps of 4.
+// = up to three tiles of 16 values of m2, reduction over the up to 16 rows of the unit in steps of 4.
 // Work-groups of eight waves: waves 0-3 keep the slot-1 gradient on the vector ALUs exactly as in
 // cg_backward_unit_kernel, waves 4-7 take slot 2 here, each every fourth m.  The two halves use
 // different pipelines of the same SIMDs (a wave of either half on each), so the vector ALUs carry
@@ -952,6 +952,7 @@ constexpr int kHybThreads = 512;
 constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
                                     // slot-2 gradient) slot 2 on the matrix cores
 constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
+constexpr int kHybMaxTiles = 3;     // 16-column tiles of the m2 axis: degrees up to 23
 // Plan: weight of a vector-ALU step of slot 1 against the matrix-core cost of slot 2 in the same
 // work-group.  Measured, not derived: below one because the matrix waves also wait on their operand
 // loads, so a unit is better off with one vector wave fewer than the instruction counts suggest.
@@ -967,7 +968,7 @@ constexpr double kHybSlot1Scale = 0.6;
 template <int NK, int NT, bool KFULL>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
-                                            int split, int lane, f32x4 (&dre)[2], f32x4 (&dim)[2]) {
+                                            int split, int lane, f32x4 (&dre)[kHybMaxTiles], f32x4 (&dim)[kHybMaxTiles]) {
     const int l = q.l, l1 = q.l1, l2 = q.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = q.rows, tau2 = q.tau2;
@@ -1022,7 +1023,7 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
         for (int c = 0; c < NK; ++c) ngy[c] = -gq[c].y;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const float cv = (NT == 2 && t == 0) || colok[t] ? cc[t] : 0.f;   // two tiles: the first one is full
+            const float cv = (t + 1 < NT) || colok[t] ? cc[t] : 0.f;   // every tile before the last one is full
 #pragma unroll
             for (int c = 0; c < NK; ++c) {
                 const float w = KFULL ? cv : cv * kmask[c];   // KFULL: the rows fill every step of four
@@ -1037,11 +1038,11 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
 }
 
 // Stores the wave's accumulator tiles: rows = channels, columns of an m axis of length Mo.
-__device__ __forceinline__ void bwd_mm_store(const f32x4 (&dre)[2], const f32x4 (&dim)[2], int n_out, int Mo, int lane,
+__device__ __forceinline__ void bwd_mm_store(const f32x4 (&dre)[kHybMaxTiles], const f32x4 (&dim)[kHybMaxTiles], int n_out, int Mo, int lane,
                                              float2* __restrict__ dst) {
     const int j = lane & 15, kk = lane >> 4;
 #pragma unroll
-    for (int tile = 0; tile < 2; ++tile) {
+    for (int tile = 0; tile < kHybMaxTiles; ++tile) {
         const int col = 16 * tile + j;
         if (col < Mo) {
 #pragma unroll
@@ -1055,9 +1056,9 @@ __device__ __forceinline__ void bwd_mm_store(const f32x4 (&dre)[2], const f32x4 
 
 __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit& u, BwdUTask t, int part, int split,
                                                   int lane, float2* __restrict__ part2_b) {
-    f32x4 dre[2], dim[2];
+    f32x4 dre[kHybMaxTiles], dim[kHybMaxTiles];
 #pragma unroll
-    for (int k = 0; k < 2; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < kHybMaxTiles; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
     int par = 0, f2par = 0;
     for (int ti = u.task_begin; ti < u.task_end; ++ti) {
         BwdUTask cur;
@@ -1066,28 +1067,20 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
 #define CGNET_MM_CALL(NK_, NT_, KF_) bwd_mm_task<NK_, NT_, KF_>(q, cgp, g, c.f1, part, split, lane, dre, dim)
+#define CGNET_MM_NT(NK_, NT_)                                           \
+    if (u.rows & 3) CGNET_MM_CALL(NK_, NT_, false);                     \
+    else CGNET_MM_CALL(NK_, NT_, true);
 #define CGNET_MM(NK_)                                                   \
-    case NK_:                                                           \
-        if (cur.l2 <= 7) {                                              \
-            if (u.rows & 3) CGNET_MM_CALL(NK_, 1, false);               \
-            else CGNET_MM_CALL(NK_, 1, true);                           \
-        } else {                                                        \
-            if (u.rows & 3) CGNET_MM_CALL(NK_, 2, false);               \
-            else CGNET_MM_CALL(NK_, 2, true);                           \
-        }                                                               \
-        break;
+    if (cur.l2 <= 7) { CGNET_MM_NT(NK_, 1) }                            \
+    else if (cur.l2 <= 15) { CGNET_MM_NT(NK_, 2) }                      \
+    else { CGNET_MM_NT(NK_, 3) }
         switch ((u.rows + 3) >> 2) {
-            CGNET_MM(1) CGNET_MM(2) CGNET_MM(3)
-            default:
-                if (cur.l2 <= 7) {
-                    if (u.rows & 3) CGNET_MM_CALL(4, 1, false);
-                    else CGNET_MM_CALL(4, 1, true);
-                } else {
-                    if (u.rows & 3) CGNET_MM_CALL(4, 2, false);
-                    else CGNET_MM_CALL(4, 2, true);
-                }
-                break;
+            case 1: CGNET_MM(1) break;
+            case 2: CGNET_MM(2) break;
+            case 3: CGNET_MM(3) break;
+            default: CGNET_MM(4) break;
         }
+#undef CGNET_MM_NT
 #undef CGNET_MM_CALL
 #undef CGNET_MM
         if (cur.last_of_l2) {
@@ -1095,7 +1088,7 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
             mfma_drain();
             bwd_mm_store(dre, dim, cur.tau2, M2, lane, part2_b + cur.p2off + (size_t)part * cur.tau2 * M2);
 #pragma unroll
-            for (int k = 0; k < 2; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < kHybMaxTiles; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
     }
 }
@@ -1461,8 +1454,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             cgp_off[i + 1] = cgp_off[i] + (int)len;
         }
         // Slot 2 on the matrix cores: needs every channel count to fit one 16-row tile (and to fill a
-        // good part of it), the m2 axis two 16-column tiles.  CGNET_BWD_HYBRID=0 keeps all on the vector ALUs.
-        bool hybrid = attempt == 0 && n1 - 1 <= 15;
+        // good part of it), the m2 axis kHybMaxTiles 16-column tiles.  CGNET_BWD_HYBRID=0 keeps all on the vector ALUs.
+        bool hybrid = attempt == 0 && n1 - 1 <= 8 * kHybMaxTiles - 1;
         for (int l = 0; l < n1; ++l)
             if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) hybrid = false;
         if (const char* e = getenv("CGNET_BWD_HYBRID"); e && e[0] == '0') hybrid = false;

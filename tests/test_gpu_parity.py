@@ -98,6 +98,8 @@ CG_CASES = [
     (11, [5] * 12, 6, "default"),                         # benchmark configuration 2 shape, small batch
     (11, [12] * 12, 3, "default"),                        # benchmark configuration 3 shape, small batch
     (15, [16] * 16, 2, "mst"),                            # benchmark configuration 4 shape, small batch
+    (17, [8] * 18, 1, "mst"),                             # degrees above 15: three column tiles in the matrix-core backward
+    (16, [9, 8, 10, 8, 12, 8, 9, 8, 16, 8, 8, 11, 8, 8, 13, 8, 10], 2, "default"),
 ]
 
 
