@@ -315,6 +315,7 @@ class CG_woFilter_cuda(nn.Module):
 
 # --------------------------------------------------------------------------- the whole layer
 _OVERLAP_GRAD_W = int(os.environ.get("CGNET_OVERLAP_GW", "1"))
+_CU_LDS_BYTES = 160 * 1024
 _side_streams = {}
 
 
@@ -361,9 +362,11 @@ class _CGBN_fused(torch.autograd.Function):
         grad_F = None
         if need_F and need_W and _OVERLAP_GRAD_W:
             # The weight gradient depends on nothing the other chain produces: it runs on a second
-            # stream (default priority) beside grad FF -> CG backward and is joined at the end.  What
-            # it gains comes from the overlap with the grad FF kernel (one reads FF, the other writes
-            # gFF); CGNET_OVERLAP_GW=0 keeps the whole backward on one stream.
+            # stream (default priority) beside grad FF.  Its tail may run into the CG backward only
+            # when one of its work-groups fits into the LDS two groups of that kernel leave on a
+            # compute unit (160 KB); otherwise the two kernels take turns on the compute units and
+            # the CG backward loses more than the overlap gains, so the side stream is joined first.
+            # CGNET_OVERLAP_GW=0 keeps the whole backward on one stream.
             main = torch.cuda.current_stream(Fs.device)
             side = _side_stream(Fs.device)
             side.wait_stream(main)
@@ -371,6 +374,8 @@ class _CGBN_fused(torch.autograd.Function):
                 ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
             ctx.wmm_plan.backward(grad_output, grad_FF, None, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
             grad_F = torch.empty_like(Fs)
+            if 2 * ctx.cg_plan.backward_lds + ctx.wmm_plan.gradw_lds > _CU_LDS_BYTES:
+                main.wait_stream(side)
             ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
             main.wait_stream(side)
             return grad_F, grad_W, None, None, None, None, None, None, None

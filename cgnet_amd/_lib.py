@@ -40,6 +40,8 @@ SIGNATURES = {
     "cgnet_FN_WMM_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_FN_WMM_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                              ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
+    "cgnet_wmm_plan_gradw_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_profile_enable": (ctypes.c_int, [ctypes.c_int]),
     "cgnet_profile_select": (ctypes.c_int, [ctypes.c_char_p]),
     "cgnet_profile_reset": (ctypes.c_int, []),

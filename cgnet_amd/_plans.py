@@ -80,6 +80,7 @@ class CGPlan:
         _lib.check(lib.cgnet_cg_plan_channels(self._h, tff, toffs))
         self.t_FF = [int(v) for v in tff]
         self.t_offsets = [int(v) for v in toffs][:len(self.llls)]
+        self.backward_lds = int(lib.cgnet_cg_plan_backward_lds(self._h))   # bytes per work-group of the backward
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -147,6 +148,7 @@ class WMMPlan:
         sizes = (ctypes.c_int * 4)()
         _lib.check(lib.cgnet_wmm_plan_sizes(self._h, sizes))
         self.nFF, self.nO, self.nW, self.sum_tFF = [int(v) for v in sizes]
+        self.gradw_lds = int(lib.cgnet_wmm_plan_gradw_lds(self._h))        # bytes per work-group of the weight gradient
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

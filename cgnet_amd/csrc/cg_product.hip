@@ -1727,6 +1727,11 @@ extern "C" int cgnet_cg_plan_sizes(const cgnet_cg_plan* plan, int sizes[5]) {
     return CGNET_OK;
 }
 
+extern "C" size_t cgnet_cg_plan_backward_lds(const cgnet_cg_plan* plan) {
+    if (!plan) return 0;
+    return plan->bwd_fast ? plan->bwd_fast_lds : plan->bwd_lds;
+}
+
 extern "C" int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, int* h_t_offsets) {
     clear_error();
     CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");

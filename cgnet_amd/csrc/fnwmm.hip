@@ -940,6 +940,11 @@ extern "C" int cgnet_wmm_plan_destroy(cgnet_wmm_plan* plan) {
     return CGNET_OK;
 }
 
+extern "C" size_t cgnet_wmm_plan_gradw_lds(const cgnet_wmm_plan* plan) {
+    if (!plan) return 0;
+    return sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
+}
+
 extern "C" int cgnet_wmm_plan_sizes(const cgnet_wmm_plan* plan, int sizes[4]) {
     clear_error();
     CGNET_REQUIRE(plan && sizes, CGNET_ERR_ARG, "null pointer argument");

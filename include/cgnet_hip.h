@@ -78,6 +78,10 @@ int cgnet_cg_plan_destroy(cgnet_cg_plan* plan);
 int cgnet_cg_plan_sizes(const cgnet_cg_plan* plan, int sizes[5]);
 /* h_t_FF[L+1], h_t_offsets[nllls]; either may be NULL */
 int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, int* h_t_offsets);
+/* LDS bytes one work-group of the product's backward kernel holds (0 without a plan).  No counterpart in the
+ * reference: a scheduling hint for callers that run another kernel on a second stream beside the backward
+ * (a compute unit has 160 KB; what two such groups leave decides whether the other kernel fits beside them). */
+size_t cgnet_cg_plan_backward_lds(const cgnet_cg_plan* plan);
 
 /* FF = CG product of F with itself over the plan's triples:
  *   FF[b, l, t_off + t1*t_F[l2] + t2, m] = sum_{m1+m2=m} CG * F[b,l1,t1,m1] * F[b,l2,t2,m2].
@@ -113,6 +117,9 @@ int cgnet_wmm_plan_create(cgnet_wmm_plan** plan, int L, const int* h_t_FF, const
 int cgnet_wmm_plan_destroy(cgnet_wmm_plan* plan);
 /* sizes[0..3] = nFF, nO, nW, sum_l t_FF[l] */
 int cgnet_wmm_plan_sizes(const cgnet_wmm_plan* plan, int sizes[4]);
+/* LDS bytes one work-group of the weight-gradient kernel holds (0 without a plan); a scheduling hint like
+ * cgnet_cg_plan_backward_lds, no counterpart in the reference. */
+size_t cgnet_wmm_plan_gradw_lds(const cgnet_wmm_plan* plan);
 
 /* O[b,l,to,m] = sum_c W[l,to,c] * FF[b,l,c,m] / max(eps, stds[c])   (no division without
  * CGNET_FN_BATCHNORM).  With CGNET_FN_UPDATE_STD the running stds are first updated in place:
