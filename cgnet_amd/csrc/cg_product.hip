@@ -77,6 +77,8 @@ struct cgnet_cg_plan {
     std::vector<int> bwd_group_table_off;        // for ng groups: first entry of its ng+1 boundaries
     int* d_bwd_group_table = nullptr;
     size_t fwd_lds = 0, bwd_lds = 0;
+    std::vector<int> fwd_class_begin;            // forward tasks by LDS class: class k = tasks [begin[k], begin[k+1])
+    std::vector<size_t> fwd_class_lds;           // LDS bytes of a work-group of class k
     int bwd_threads = 256;                       // work-group size of the backward kernel
     // register-resident backward (used when every unit fits; otherwise the LDS-accumulator kernel)
     bool bwd_fast = false;
@@ -1389,6 +1391,22 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         return (long long)a.rows * a.tau2 * (2 * a.l + 1) * (2 * a.l2 + 1) >
                (long long)b.rows * b.tau2 * (2 * b.l + 1) * (2 * b.l2 + 1);
     });
+    // One launch has one LDS size, and the largest task's would set the occupancy of all: the tasks are
+    // grouped by the number of work-groups per compute unit their own LDS need allows (at most four, the
+    // register limit), largest need first, and every class gets a launch of its own.
+    auto fwd_class = [](const CgTask& t) { return (int)std::max<size_t>(1, std::min<size_t>(4, kMaxLds / align_up(fwd_task_lds(t), 16))); };
+    std::stable_sort(p->fwd_tasks.begin(), p->fwd_tasks.end(),
+                     [&](const CgTask& a, const CgTask& b) { return fwd_class(a) < fwd_class(b); });
+    p->fwd_class_begin.clear();
+    p->fwd_class_lds.clear();
+    for (size_t k = 0; k < p->fwd_tasks.size(); ++k) {
+        if (k == 0 || fwd_class(p->fwd_tasks[k]) != fwd_class(p->fwd_tasks[k - 1])) {
+            p->fwd_class_begin.push_back((int)k);
+            p->fwd_class_lds.push_back(0);
+        }
+        p->fwd_class_lds.back() = std::max(p->fwd_class_lds.back(), align_up(fwd_task_lds(p->fwd_tasks[k]), 16));
+    }
+    p->fwd_class_begin.push_back((int)p->fwd_tasks.size());
     size_t fl = 0, bl = 0;
     for (const CgTask& t : p->fwd_tasks) {
         fl = std::max(fl, fwd_task_lds(t));
@@ -1747,9 +1765,13 @@ static int launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF,
     const int ngroups = (B + spg - 1) / spg;
     CGNET_REQUIRE((long long)ntasks * ngroups < (1LL << 31), CGNET_ERR_UNSUPPORTED,
                   "%d tasks x %d sample groups exceed the grid limit", ntasks, ngroups);
-    CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(ntasks * ngroups)), dim3(kThreads), p->fwd_lds, s,
-                       (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks, p->nF, p->nFF, B, spg, d_part, p->sumT);
-    CGNET_HIP(hipGetLastError());
+    for (size_t k = 0; k + 1 < p->fwd_class_begin.size(); ++k) {
+        const int t0 = p->fwd_class_begin[k], nt = p->fwd_class_begin[k + 1] - t0;
+        CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(nt * ngroups)), dim3(kThreads), p->fwd_class_lds[k], s,
+                           (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
+                           p->sumT);
+        CGNET_HIP(hipGetLastError());
+    }
     return CGNET_OK;
 }
 
