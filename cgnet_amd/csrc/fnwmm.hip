@@ -573,26 +573,31 @@ __global__ void __launch_bounds__(256)
 pack_w_gradff_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                      const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Ap, int total_blocks) {
     __shared__ int s_tab[kMaxLookup];
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // one weight = two packed floats
-    const int blk = idx >> 5, half = (idx >> 4) & 1, i = idx & 15;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // four weights of one row = two 16-byte stores
+    const int blk = idx >> 3, half = (idx >> 2) & 1, i0 = (idx & 3) * 4;
     const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].ap_base; }, s_tab);
     if (blk >= total_blocks) return;
     const WmmDeg d = degs[di];
     const int rel = blk - d.ap_base;             // ctile * nks_b + ks
     const int ks = rel % d.nks_b, ctile = rel / d.nks_b;
-    const int c = ctile * 16 + i, to = 2 * ks + half;             // k = 4*ks + kk, to = k >> 1, kk = 2*half + sel
-    float2 w = make_float2(0.f, 0.f);
-    if (c < d.K && to < d.tO) {
-        w = W[d.cumW + (size_t)to * d.K + c];
-        if (stds) {
-            const float r = fmaxf(eps, stds[d.cumT + c]);
-            w.x /= r;
-            w.y /= r;
+    const int c0 = ctile * 16 + i0, to = 2 * ks + half;           // k = 4*ks + kk, to = k >> 1, kk = 2*half + sel
+    float re[4] = {0.f, 0.f, 0.f, 0.f}, im[4] = {0.f, 0.f, 0.f, 0.f};
+    if (to < d.tO) {
+        const float2* wrow = W + d.cumW + (size_t)to * d.K;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + j;
+            if (c < d.K) {
+                const float2 w = wrow[c];
+                const float r = stds ? fmaxf(eps, stds[d.cumT + c]) : 1.f;
+                re[j] = stds ? w.x / r : w.x;
+                im[j] = stds ? w.y / r : w.y;
+            }
         }
     }
-    float* dst = Ap + (size_t)blk * 64 + half * 32 + i;
-    dst[0] = w.x;
-    dst[16] = w.y;
+    float* dst = Ap + (size_t)blk * 64 + half * 32 + i0;
+    *reinterpret_cast<float4*>(dst) = make_float4(re[0], re[1], re[2], re[3]);
+    *reinterpret_cast<float4*>(dst + 16) = make_float4(im[0], im[1], im[2], im[3]);
 }
 
 // Gradient with respect to FF on the matrix cores (t_O <= 16): gFF[c, (m, re/im)] = sum_k A[c, k] * B[k, (m, re/im)]
@@ -1106,7 +1111,7 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
         CGNET_REQUIRE(plan->nO == 0 || d_gO, CGNET_ERR_ARG, "d_gO is NULL");
         if (plan->gff_mfma && plan->nW > 0 && plan->nO > 0) {
             float* Ap = (float*)d_workspace;
-            const int total = plan->ap_blocks * 32;   // one thread per weight
+            const int total = plan->ap_blocks * 8;    // one thread per four weights
             CGNET_LAUNCH(pack_w_gradff_kernel, dim3((total + 255) / 256), dim3(256), 0, s, (const float2*)d_W,
                          bn ? d_stds : nullptr, eps, plan->d_degs, ndeg, Ap, plan->ap_blocks);
             CGNET_HIP(hipGetLastError());
