@@ -39,6 +39,55 @@ def synthetic(lmax, tau, bsz, t_ff, seed=0):
     return x, w, go
 
 
+TRAFFIC_PROFILE = os.path.join("profiles", "cg_layer_L11_tau12_B100_hbm_traffic_pmc.txt")
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the streaming kernels as the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
+    summary states them (counters are not readable from inside a run; the summary names the command and
+    the source revision it was measured on).  -> ({kernel: bytes}, description of the source)."""
+    import re
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    table, rev = {}, "unknown revision"
+    try:
+        for line in open(path):
+            m = re.match(r"^(\w+)(?:<\d+>)?\s+([\d.]+) MB\s+([\d.]+) MB\s+([\d.]+) MB\s+([\d.]+) MB\s+[\d.]+\s*$", line)
+            if m:
+                table[m.group(1)] = float(m.group(4)) * 1e6
+            m = re.match(r"^source revision:\s*(\S+)", line)
+            if m:
+                rev = m.group(1)
+    except OSError:
+        return {}, "no traffic profile found"
+    return table, "%s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; measured at %s, not in this run)" % (TRAFFIC_PROFILE, rev)
+
+
+def host_cpu():
+    """(model name, physical cores, logical cpus) of the host, from /proc/cpuinfo."""
+    model, cores, logical = "unknown", set(), 0
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "processor":
+                logical += 1
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None:
+                cores.add((phys, core))
+                phys = core = None
+        if phys is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    return model, (len(cores) or logical), logical
+
+
 def cpu_baseline(lmax, tau, codes, t_ff, sample_batch, repeats):
     """The oracle's float32 layer (port of the reference's python path) on the host cores."""
     import numpy as np
@@ -60,10 +109,13 @@ def cpu_baseline(lmax, tau, codes, t_ff, sample_batch, repeats):
     for _ in range(repeats):
         step()
     dt = (time.perf_counter() - t0) / repeats
+    model, physical, logical = host_cpu()
     return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(torch.get_num_threads()),
-            "kind": "port",
-            "sample": "B=%d of the same L=%d tau=%d layer fwd+bwd, float32 torch CPU oracle, 1 warm-up + %d timed "
-                      "steps, %.1f s per step" % (sample_batch, lmax, tau, repeats, dt)}
+            "kind": "port", "cpu_model": model, "physical_cores": physical, "logical_cpus": logical,
+            "threads_used": int(torch.get_num_threads()), "cpu_batch": sample_batch, "gpu_batch": WORKLOAD["batch"],
+            "sample": "B=%d (the GPU line runs B=%d) of the same L=%d tau=%d layer fwd+bwd, float32 torch CPU oracle, "
+                      "1 warm-up + %d timed steps, %.1f s per step; the per-sample cost of the oracle does not depend "
+                      "on B" % (sample_batch, WORKLOAD["batch"], lmax, tau, repeats, dt)}
 
 
 def main():
@@ -118,6 +170,12 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # untimed: keep the GPU busy for a moment so that the timed steps run at the settled clock, whatever W was
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < 0.4:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     # untimed survey with every kernel bracketed by events: per-kernel table, and which kernel dominates
     lib.cgnet_profile_reset()
     lib.cgnet_profile_select(None)
@@ -163,12 +221,7 @@ def main():
         "cg_backward_hybrid_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
-    # HBM bytes per launch at this workload from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
-    # profiles/cg_layer_L11_tau12_B100_hbm_traffic_pmc.txt (calibrated against a copy kernel of known size)
-    measured_traffic = {
-        "cg_backward_hybrid_kernel": 809.9e6, "cg_forward_kernel": 796.1e6, "wmm_forward_kernel": 925.2e6,
-        "wmm_gradw_kernel": 807.5e6, "wmm_gradff_mfma_kernel": 832.5e6,
-    }
+    measured_traffic, traffic_source = profiled_traffic()
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
     kernels = {}
     for name, (ms, cnt) in sorted(survey.items(), key=lambda kv: -kv[1][0]):
@@ -194,6 +247,7 @@ def main():
                    "lmax": lmax, "tau": tau, "batch": bsz, "triples": len(layer.cg.lll_list)},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic.get(dominant),
+                     "traffic_source": traffic_source,
                      "algorithmic_bytes_per_launch": algo[dominant], "avg_launch_ms": d_avg_s * 1e3},
         "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
                        "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},

@@ -68,6 +68,30 @@ def load_normalisation_counts(module, counts):
         named[name].bn_cnt = float(cnt)
 
 
-# The reference's README and Shrec17 script name a "SphericalCNN_fast"; its source is not part
-# of the reference, so only the name can be honoured.
-SphericalCNN_fast = SphericalCNN
+class SphericalCNN_fast(SphericalCNN):
+    """The stack under the constructor the reference's Shrec17 script calls
+    (Shrec17/Shrec17_main_fast.py:78-79): ``SphericalCNN(lmax, taus, nlayers, skip_type=, num_channels_input=)``
+    with ``taus`` ONE list of channels per degree shared by all layers.  The class itself is not part of the
+    reference (the script imports it from a module the repository does not hold), so the meaning of the
+    arguments is taken from that call site and from ``SphericalCNN``:
+
+    * the input carries ``num_channels_input`` channels in every degree (6 spherical signals per SHREC17 mesh);
+    * ``nlayers`` layers follow, each producing ``taus``;
+    * ``skip_type`` 0 returns the last layer's l=0 fragment only, 1 the concatenation of the l=0 fragments of the
+      input and of every layer (``skipconn``); the script routes other values to residual classes that are not
+      in the reference either, and they are refused here.
+    """
+
+    def __init__(self, lmax, taus, nlayers, skip_type=1, num_channels_input=1, norm=True, sparse_flag=False,
+                 device=None):
+        if skip_type not in (0, 1):
+            raise NotImplementedError("skip_type=%r: only 0 (last l=0 fragment) and 1 (skip connections) exist" % (skip_type,))
+        if len(taus) != lmax + 1:
+            raise AssertionError("taus must have lmax+1 entries")
+        if int(nlayers) < 1 or int(num_channels_input) < 1:
+            raise AssertionError("nlayers and num_channels_input must be positive")
+        per_layer = [[int(num_channels_input)] * (lmax + 1)] + [[int(t) for t in taus] for _ in range(int(nlayers))]
+        super().__init__(lmax, per_layer, cuda=True, norm=norm, skipconn=bool(skip_type), sparse_flag=sparse_flag,
+                         device=device)
+        self.skip_type = skip_type
+        self.num_channels_input = int(num_channels_input)

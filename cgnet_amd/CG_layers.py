@@ -140,8 +140,23 @@ class MyBatchNormWeightMM_cuda(nn.Module):
             self.bn_cnt += 1
         return output
 
-    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
-        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+    # ``bn_cnt`` stays the plain float attribute of the reference (CG_layers.py:92,130: read on every forward, so
+    # it must not live on the device), but unlike there it travels with ``state_dict`` as the entry ``bn_cnt``,
+    # so a resumed run continues the moving average where it stopped.  Checkpoints written by the reference lack
+    # the entry: loading them keeps the current count.
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        destination[prefix + "bn_cnt"] = torch.tensor(float(self.bn_cnt), dtype=torch.float64)
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        key = prefix + "bn_cnt"
+        cnt = state_dict.pop(key, None) if key in state_dict else None
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+        if cnt is not None:
+            self.bn_cnt = float(cnt)
+            state_dict[key] = cnt          # the caller's dictionary is left as it was
         self._eps_host = float(self.bn_eps.detach().cpu().item())
 
 

@@ -1716,14 +1716,12 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         CGNET_HIP(hipMemcpy(p->d_bwd_combine, combine_meta.data(), sizeof(int) * combine_meta.size(), hipMemcpyHostToDevice));
         CGNET_HIP(hipMalloc((void**)&p->d_bwd_padmeta, sizeof(int) * pad_meta.size()));
         CGNET_HIP(hipMemcpy(p->d_bwd_padmeta, pad_meta.data(), sizeof(int) * pad_meta.size(), hipMemcpyHostToDevice));
-        if (p->bwd_fast_lds > 64 * 1024)
-            CGNET_HIP(hipFuncSetAttribute(p->bwd_hybrid ? (const void*)cg_backward_hybrid_kernel : (const void*)cg_backward_unit_kernel,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_fast_lds));
+        if (int rc = raise_dynamic_lds(p->bwd_hybrid ? (const void*)cg_backward_hybrid_kernel : (const void*)cg_backward_unit_kernel,
+                                       p->bwd_fast_lds))
+            return rc;
     }
-    if (p->fwd_lds > 64 * 1024)
-        CGNET_HIP(hipFuncSetAttribute((const void*)cg_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->fwd_lds));
-    if (p->bwd_lds > 64 * 1024)
-        CGNET_HIP(hipFuncSetAttribute((const void*)cg_backward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)p->bwd_lds));
+    if (int rc = raise_dynamic_lds((const void*)cg_forward_kernel, p->fwd_lds)) return rc;
+    if (int rc = raise_dynamic_lds((const void*)cg_backward_kernel, p->bwd_lds)) return rc;
     *plan = guard.release();
     return CGNET_OK;
 }

@@ -35,6 +35,12 @@ constexpr int kMaxTau = 1024;      // channels of one degree
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Makes sure `func` may be launched with `bytes` of dynamic LDS on the current device.  The
+// attribute is per kernel and device, not per plan: the largest size any plan of this process has
+// asked for is kept and only ever raised, so plans with different needs can be launched in any order.
+// Returns CGNET_OK or CGNET_ERR_HIP (message recorded).
+int raise_dynamic_lds(const void* func, size_t bytes);
+
 // Optional per-kernel timing (cgnet_profile_*): when enabled, every launch is bracketed by a
 // pair of HIP events recorded on the launch stream.
 class KernelTimer {

@@ -19,6 +19,20 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 void clear_error() { g_err[0] = 0; }
+
+int raise_dynamic_lds(const void* func, size_t bytes) {
+    static std::mutex mu;
+    static std::map<std::pair<const void*, int>, size_t> granted;
+    if (bytes <= 64 * 1024) return CGNET_OK;          // the default limit covers it
+    int device = 0;
+    CGNET_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(mu);
+    size_t& have = granted[std::make_pair(func, device)];
+    if (bytes <= have) return CGNET_OK;
+    CGNET_HIP(hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    have = bytes;
+    return CGNET_OK;
+}
 }  // namespace cgnet
 
 extern "C" const char* cgnet_last_error(void) { return cgnet::g_err; }

@@ -74,7 +74,8 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kStatTileBytes = 32 * 1024;
 constexpr int kStatGroups = 8;
-constexpr int kGradWChunk = 32;     // samples accumulated in one matrix-core chain of the weight gradient
+constexpr int kGradWChunk = 32;     // samples whose weight-gradient sums one work-group forms
+constexpr int kGradWFold = 4;       // samples per matrix-core chain inside a chunk
 
 // --------------------------------------------------------------------------- statistics
 // sums of |z| and |z|^2 over (b, m) per mid channel, from FF
@@ -246,6 +247,7 @@ __device__ __forceinline__ void wmm_forward_wave(const float2* __restrict__ FF, 
         // never writes are multiplied by zero weights or land in columns nobody stores
         float4* z = reinterpret_cast<float4*>(ring);
         for (int e = lane; e < (depth * stage_bytes) >> 4; e += 64) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the clearing stores precede the first copy into the ring
     }
     const int nk = u.k_end - u.k_begin;
     const int nfull = nk / kFwdKC, nstages = (nk + kFwdKC - 1) / kFwdKC;
@@ -470,8 +472,12 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
         if (n_go & 1) dma8(gsrc + (n_go - 1), gdst + (n_go - 1), tid);
     };
     if (b_begin < b_end) issue(b_begin, 0);
+    // Blocked summation: the matrix-core chain runs over kGradWFold samples, then its sums are folded into
+    // the totals -- a chain over the whole chunk (32 samples x 2M terms) loses several times the digits of the
+    // blocked sums of a CPU matrix product.
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    int buf = 0;
+    f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
+    int buf = 0, since = 0;
     for (int b = b_begin; b < b_end; ++b, buf ^= 1) {
         const float2* ffl = ffbuf + buf * ff_cap;
         const float2* gol = gobuf + buf * go_cap;
@@ -494,15 +500,24 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
                     }
                     break;
             }
+            if (++since == kGradWFold) {
+                since = 0;
+                mfma_drain();
+                tot0 += acc0;
+                tot1 += acc1;
+                acc0 = acc1 = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
         }
     }
     mfma_drain();
+    tot0 += acc0;
+    tot1 += acc1;
     if (cok) {
         float2* dst = part + (size_t)up.part * nW;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int to = u.rc * 16 + 4 * kk + v;
-            if (to < d.tO) dst[d.cumW + (size_t)to * d.K + c] = make_float2(acc0[v], acc1[v]);
+            if (to < d.tO) dst[d.cumW + (size_t)to * d.K + c] = make_float2(tot0[v], tot1[v]);
         }
     }
 }

@@ -1,13 +1,23 @@
 """GPU parity tests: every native entry point against the CPU oracle on the same seeded inputs.
 
-Tolerance (the north star's fp32 bar): |gpu - oracle64| <= 1e-6 * max(1, max|oracle64|) + 1e-5 * |oracle64|
-elementwise, where oracle64 is the float64 evaluation of the reference's python algorithm.  The
-absolute term is expressed in units of the tensor's largest entry once that exceeds 1, because
-float32 cannot resolve 1e-6 on sums whose terms have magnitude >> 1 (weight gradients and
-normalised channels with a small running std reach ~1e2; an entry that cancels to ~0 there still
-carries the rounding error of its large terms, for the float32 CPU path as much as for the GPU).
+Tolerance.  The north star's bar is elementwise  |gpu - oracle64| <= 1e-6 + 1e-5 * |oracle64|  with oracle64 the
+float64 evaluation of the reference's python algorithm on float32-representable inputs.  Single precision
+cannot hold that bar on sums whose terms are much larger than the result (weight gradients and channels
+normalised by a small running std reach 1e2; an entry that cancels to ~0 still carries the rounding of
+its large terms).  How much of that is the arithmetic's and how much the GPU's is measured, not assumed: every
+comparison also evaluates the oracle in float32 on the CPU (the reference's own precision), and the GPU
+must satisfy
+
+    |gpu - oracle64|  <=  max( 1e-6 + 1e-5 * |oracle64| ,  4 * max|cpu32 - oracle64| )      elementwise,
+
+i.e. it is held to the strict bar wherever the float32 CPU path itself meets it, and otherwise to four times that
+path's worst error on the same tensor (the CPU path sums through BLAS in blocks, the kernels in chains of up to a
+few hundred terms, so worst-case errors two to three times the CPU's are the order of summation, not a defect).  Both maxima are printed (``pytest -s``) and, when the
+environment variable CGNET_PARITY_REPORT names a file, appended to it as JSON lines.
 """
+import json
 import math
+import os
 
 import numpy as np
 import pytest
@@ -20,6 +30,8 @@ from oracle import triples as OT
 pytestmark = pytest.mark.gpu
 
 RTOL, ATOL = 1e-5, 1e-6
+TWIN_FACTOR = 4.0
+F64, F32 = torch.float64, torch.float32
 
 
 @pytest.fixture(scope="module")
@@ -31,19 +43,37 @@ def dev():
     return torch.device("cuda:0")
 
 
-def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
-    got = got.detach().double().cpu().reshape(-1)
-    ref = ref.detach().double().cpu().reshape(-1)
+def _flat(t):
+    return t.detach().double().cpu().reshape(-1)
+
+
+def assert_close(got, ref, what, twin=None, rtol=RTOL, atol=ATOL):
+    """``ref``: float64 oracle; ``twin``: the same oracle evaluated in float32 on the CPU (None: strict bar only)."""
+    got, ref = _flat(got), _flat(ref)
     assert got.shape == ref.shape, what
     assert torch.isfinite(got).all(), what + ": non-finite values"
-    rms = float(ref.abs().max()) if ref.numel() else 0.0
-    bound = atol * max(1.0, rms) + rtol * ref.abs()
+    if ref.numel() == 0:
+        return
+    strict = atol + rtol * ref.abs()
     err = (got - ref).abs()
-    worst = int(torch.argmax(err - bound)) if ref.numel() else 0
+    err_twin = float((_flat(twin) - ref).abs().max()) if twin is not None else 0.0
+    bound = torch.clamp(strict, min=TWIN_FACTOR * err_twin)
+    rec = {"test": os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0], "what": what, "n": ref.numel(),
+           "max_ref": float(ref.abs().max()), "err_gpu": float(err.max()), "err_cpu32": err_twin if twin is not None else None,
+           "strict_violations_gpu": int((err > strict).sum()),
+           "strict_violations_cpu32": int(((_flat(twin) - ref).abs() > strict).sum()) if twin is not None else None}
+    print("[parity] %-28s max|ref| %.3e  err_gpu %.3e  err_cpu32 %s  outside strict bar: gpu %d cpu32 %s of %d"
+          % (what, rec["max_ref"], rec["err_gpu"], "%.3e" % err_twin if twin is not None else "-",
+             rec["strict_violations_gpu"], rec["strict_violations_cpu32"], ref.numel()))
+    path = os.environ.get("CGNET_PARITY_REPORT")
+    if path:
+        with open(path, "a") as fh:
+            fh.write(json.dumps(rec) + "\n")
+    worst = int(torch.argmax(err - bound))
     assert bool((err <= bound).all()), (
-        "%s: %d of %d outside tolerance; worst |err|=%.3e at %d (ref %.6e, bound %.3e, max|ref| %.3e)"
+        "%s: %d of %d outside tolerance; worst |err|=%.3e at %d (ref %.6e, bound %.3e, cpu32 max err %.3e)"
         % (what, int((err > bound).sum()), ref.numel(), float(err[worst]), worst, float(ref[worst]),
-           float(bound[worst]), rms))
+           float(bound[worst]), err_twin))
 
 
 def make_codes(lmax, mode):
@@ -64,7 +94,11 @@ def rand_straight(taus, bsz, seed, scaled=True):
     for l, t in enumerate(taus):
         x = torch.randn(bsz, t * (2 * l + 1), 2, generator=g, dtype=torch.float64)
         parts.append(x / math.sqrt(2 * l + 1) if scaled else x)
-    return torch.cat(parts, dim=1)
+    return torch.cat(parts, dim=1).float().double()       # representable in float32: GPU and oracle see the same numbers
+
+
+def randn32(shape, gen):
+    return torch.randn(shape, generator=gen, dtype=torch.float64).float().double()
 
 
 # ------------------------------------------------------------------------------- CG table
@@ -100,15 +134,17 @@ CG_CASES = [
     (15, [16] * 16, 2, "mst"),                            # benchmark configuration 4 shape, small batch
     (17, [8] * 18, 1, "mst"),                             # degrees above 15: three column tiles in the matrix-core backward
     (16, [9, 8, 10, 8, 12, 8, 9, 8, 16, 8, 8, 11, 8, 8, 13, 8, 10], 2, "default"),
+    (20, [16] * 21, 1, "default"),                        # benchmark configuration 5, layers 2-4: three column tiles in the
+                                                          # matrix-core backward, two LDS classes in the forward
 ]
 
 
-def cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64=None):
-    x = x64.clone().requires_grad_(True)
+def cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64=None, dtype=F64):
+    x = x64.to(dtype).clone().requires_grad_(True)
     y = OL.join_straight(OL.cg_product(x, lmax, codes, taus))
     if gy64 is None:
         return y.detach(), None
-    (gx,) = torch.autograd.grad(y, x, gy64)
+    (gx,) = torch.autograd.grad(y, x, gy64.to(dtype))
     return y.detach(), gx
 
 
@@ -120,15 +156,16 @@ def test_cg_forward_backward(dev, lmax, taus, bsz, mode):
     mod = CG_layers.CG_woFilter_cuda(lmax, taus, lll_mode=None if mode == "default" else mode, device=dev)
     assert mod.lll_list == codes
     g = torch.Generator().manual_seed(17)
-    gy64 = torch.randn(bsz, int(mod.cumu_tm_FF[-1]), 2, generator=g, dtype=torch.float64)
+    gy64 = randn32((bsz, int(mod.cumu_tm_FF[-1]), 2), g)
     want_y, want_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64)
+    twin_y, twin_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64, dtype=F32)
 
     x = x64.float().to(dev).requires_grad_(True)
     y = mod(x, straight_output=True)
     assert y.shape == want_y.shape
-    assert_close(y, want_y, "CG forward")
+    assert_close(y, want_y, "CG forward", twin_y)
     y.backward(gy64.float().to(dev))
-    assert_close(x.grad, want_gx, "CG backward")
+    assert_close(x.grad, want_gx, "CG backward", twin_gx)
 
     # list input / list output views
     parts = OL.split_straight(x.detach(), taus)
@@ -186,12 +223,13 @@ def test_cg_backward_general_kernel(dev, monkeypatch, lmax, taus, bsz, mode):
     _plans.fill_cg_table(cg, lmax, codes, [int(v) for v in offs])
     x64 = rand_straight(taus, bsz, seed=77)
     g = torch.Generator().manual_seed(78)
-    gy64 = torch.randn(bsz, plan.nFF, 2, generator=g, dtype=torch.float64)
+    gy64 = randn32((bsz, plan.nFF, 2), g)
     _, want_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64)
+    _, twin_gx = cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64, dtype=F32)
     x = x64.float().to(dev)
     gx = torch.full_like(x, float("nan"))
     plan.backward(x, gx, gy64.float().to(dev), cg, bsz)
-    assert_close(gx, want_gx, "CG backward (general kernel)")
+    assert_close(gx, want_gx, "CG backward (general kernel)", twin_gx)
 
 
 def test_cg_forward_matches_dense_definition(dev):
@@ -227,13 +265,13 @@ def test_cg_deterministic(dev):
 
 
 # ------------------------------------------------------------------------------- fragment norm + mixing
-def wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds, eps, bn, training, cnt, go64=None):
-    ff = ff64.clone().requires_grad_(True)
-    w = w64.clone().requires_grad_(True)
+def wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds, eps, bn, training, cnt, go64=None, dtype=F64):
+    ff = ff64.to(dtype).clone().requires_grad_(True)
+    w = w64.to(dtype).clone().requires_grad_(True)
     parts = OL.split_straight(ff, t_ff)
     st, o = [], 0
     for t in t_ff:
-        st.append(np.array(stds[o:o + t], dtype=np.float64))
+        st.append(np.array(stds[o:o + t], dtype=np.float64 if dtype == F64 else np.float32))
         o += t
     if bn:
         OL.fragment_norm_update([p for p in parts], st, cnt, training)
@@ -241,7 +279,7 @@ def wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds, eps, bn, training, cnt, go64=
     out = OL.join_straight(OL.weight_mix(parts, w, t_ff, t_out))
     res = {"out": out.detach(), "stds": np.concatenate(st) if len(st) else np.zeros(0)}
     if go64 is not None:
-        gff, gw = torch.autograd.grad(out, (ff, w), go64)
+        gff, gw = torch.autograd.grad(out, (ff, w), go64.to(dtype))
         res["gFF"], res["gW"] = gff, gw
     return res
 
@@ -285,17 +323,18 @@ def test_fn_wmm_forward_backward(dev, lmax, t_ff, t_out, bsz, bn, training):
 def check_fn_wmm(dev, lmax, t_ff, t_out, bsz, bn, training):
     from cgnet_amd import CG_layers
     g = torch.Generator().manual_seed(1000 + lmax + bsz)
-    ff64 = rand_straight(t_ff, bsz, seed=5) * 0.3
+    ff64 = (rand_straight(t_ff, bsz, seed=5) * 0.3).float().double()
     n_w = sum(a * b for a, b in zip(t_ff, t_out))
     w64 = torch.cat([torch.randn(t_ff[l] * t_out[l], 2, generator=g, dtype=torch.float64) / math.sqrt(max(1, t_ff[l]))
-                     for l in range(lmax + 1)]) if n_w else torch.zeros(0, 2, dtype=torch.float64)
+                     for l in range(lmax + 1)]).float().double() if n_w else torch.zeros(0, 2, dtype=torch.float64)
     stds0 = (0.05 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64) * 0.3).float()
     if sum(t_ff) > 3:
         stds0[1] = 1e-9                                   # exercises the eps floor
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(t_out))
-    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
+    go64 = randn32((bsz, n_o, 2), g)
     cnt = 3.0
     want = wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds0.double().numpy(), 1e-5, bn, training, cnt, go64)
+    twin = wmm_oracle(lmax, t_ff, t_out, ff64, w64, stds0.double().numpy(), 1e-5, bn, training, cnt, go64, dtype=F32)
 
     mod = CG_layers.MyBatchNormWeightMM_cuda(lmax, t_ff, t_out, batchnorm=bn, device=dev)
     with torch.no_grad():
@@ -307,13 +346,13 @@ def check_fn_wmm(dev, lmax, t_ff, t_out, bsz, bn, training):
     ff = ff64.float().to(dev).requires_grad_(True)
     out = mod(ff)
     assert out.shape == (bsz, n_o, 2)
-    assert_close(out, want["out"], "WMM forward")
+    assert_close(out, want["out"], "WMM forward", twin["out"])
     if bn:
         assert_close(mod.bn_stds, torch.from_numpy(want["stds"]), "running stds", rtol=2e-6, atol=1e-8)
         assert mod.bn_cnt == (cnt + 1 if training else cnt)
     out.backward(go64.float().to(dev))
-    assert_close(ff.grad, want["gFF"], "grad FF")
-    assert_close(mod.W.grad, want["gW"], "grad W")
+    assert_close(ff.grad, want["gFF"], "grad FF", twin["gFF"])
+    assert_close(mod.W.grad, want["gW"], "grad W", twin["gW"])
 
 
 def test_gradw_deterministic(dev):
@@ -337,70 +376,111 @@ LAYER_CASES = [
     (3, [2, 2, 2, 2], [2, 2, 2, 2], 4, False, True),
     (3, [2, 2, 2, 2], [3, 1, 2, 2], 4, True, True),
     (4, [3, 2, 1, 2, 2], [2, 2, 2, 2, 2], 3, False, False),
-    (11, [5] * 12, [5] * 12, 8, False, True),            # benchmark configuration 2 shape (B reduced for the oracle)
-    (11, [12] * 12, [12] * 12, 3, False, True),          # benchmark configuration 3 shape (B reduced)
+    (11, [5] * 12, [5] * 12, 32, False, True),           # benchmark configuration 2
+    (11, [12] * 12, [12] * 12, 3, False, True),          # benchmark configuration 3 shape (B reduced for the oracle)
 ]
+
+
+def layer_weights(lmax, t_ff, tout, seed):
+    """Injected parameters (float32-representable): W ~ N(0, 1/t_FF), running stds in [0.02, 0.12)."""
+    g = torch.Generator().manual_seed(seed)
+    w64 = torch.cat([torch.randn(t_ff[l] * tout[l], 2, generator=g, dtype=torch.float64) / math.sqrt(max(1, t_ff[l]))
+                     for l in range(lmax + 1)]).float().double()
+    stds = (0.02 + 0.1 * torch.rand(sum(t_ff), generator=g, dtype=torch.float64)).float()
+    return w64, stds
+
+
+def make_oracle(lmax, tin, tout, codes, bn, stds, dtype=F64):
+    """The layer oracle in float64 (arbiter) or float32 (the reference's own precision, statistics included)."""
+    ora = OL.LayerOracle(lmax, tin, tout, codes, batchnorm=bn, eps=1e-5)
+    if bn:
+        ora.set_stds_flat(stds.numpy().astype(np.float64 if dtype == F64 else np.float32))
+    return ora
+
+
+def oracle_step(ora, x64, w64, go64, dtype=F64):
+    xo = x64.to(dtype).clone().requires_grad_(True)
+    wo = w64.to(dtype).clone().requires_grad_(True)
+    out = OL.join_straight(ora.forward(xo, wo))
+    gx, gw = torch.autograd.grad(out, (xo, wo), go64.to(dtype), allow_unused=True)
+    return out.detach(), (gx if gx is not None else torch.zeros_like(xo)), (gw if gw is not None else torch.zeros_like(wo))
 
 
 def build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed):
     from cgnet_amd import CG_layers
     mod = CG_layers.CGBN_cuda(lmax, tin, tout, batchnorm=bn, sparse_flag=sparse, device=dev)
-    codes = mod.cg.lll_list
-    ora = OL.LayerOracle(lmax, tin, tout, codes, batchnorm=bn, eps=1e-5)
-    g = torch.Generator().manual_seed(seed)
     t_ff = [int(v) for v in mod.t_FF]
-    w64 = torch.cat([torch.randn(t_ff[l] * tout[l], 2, generator=g, dtype=torch.float64) / math.sqrt(max(1, t_ff[l]))
-                     for l in range(lmax + 1)])
-    stds = 0.02 + 0.1 * torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
+    w64, stds = layer_weights(lmax, t_ff, tout, seed)
     with torch.no_grad():
         mod.bnWMM.W.copy_(w64.float())
         if bn:
-            mod.bnWMM.bn_stds.copy_(stds.float())
-    if bn:
-        ora.set_stds_flat(stds.float().double().numpy())
-    return mod, ora, w64.float().double()
+            mod.bnWMM.bn_stds.copy_(stds)
+    ora = make_oracle(lmax, tin, tout, mod.cg.lll_list, bn, stds)
+    twin = make_oracle(lmax, tin, tout, mod.cg.lll_list, bn, stds, dtype=F32)
+    return mod, ora, twin, w64
+
+
+def check_layer_step(dev, mod, ora, twin, w64, x64, go64):
+    """One training step of the layer on the GPU against the float64 oracle and its float32 twin."""
+    want, want_gx, want_gw = oracle_step(ora, x64, w64, go64)
+    tw, tw_gx, tw_gw = oracle_step(twin, x64, w64, go64, dtype=F32)
+    x = x64.float().to(dev).requires_grad_(True)
+    mod.bnWMM.W.grad = None
+    out = mod(x, straight_output=True)
+    assert_close(out, want, "layer forward", tw)
+    if ora.batchnorm:
+        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds",
+                     torch.from_numpy(twin.stds_flat().astype(np.float64)), rtol=5e-6, atol=1e-8)
+    out.backward(go64.float().to(dev))
+    assert_close(x.grad, want_gx, "layer grad F", tw_gx)
+    if w64.numel():
+        assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W", tw_gw)
+    return x
 
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn", LAYER_CASES)
 def test_layer_forward_backward(dev, lmax, tin, tout, bsz, sparse, bn, fused):
-    mod, ora, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=lmax + bsz)
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=lmax + bsz)
     mod.fused = fused
     x64 = rand_straight(tin, bsz, seed=21)
     g = torch.Generator().manual_seed(23)
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
-    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
-
-    xo = x64.float().double().requires_grad_(True)
-    wo = w64.clone().requires_grad_(True)
-    want = OL.join_straight(ora.forward(xo, wo))
-    want_gx, want_gw = torch.autograd.grad(want, (xo, wo), go64)
-
-    x = x64.float().to(dev).requires_grad_(True)
-    out = mod(x, straight_output=True)
-    assert_close(out, want, "layer forward")
+    go64 = randn32((bsz, n_o, 2), g)
+    x = check_layer_step(dev, mod, ora, twin, w64, x64, go64)
     if bn:
-        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds", rtol=5e-6, atol=1e-8)
         assert mod.bnWMM.bn_cnt == 2.0
-    out.backward(go64.float().to(dev))
-    assert_close(x.grad, want_gx, "layer grad F")
-    assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W")
-
+    if bsz > 8:
+        return                                           # the follow-up steps below repeat the oracle three times
     # second training step: the moving average advances with count 2
     if bn:
-        want2 = OL.join_straight(ora.forward(xo.detach() * 0.5, wo.detach()))
-        out2 = mod((x.detach() * 0.5), straight_output=True)
-        assert_close(out2, want2, "second step forward")
-        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds step 2", rtol=5e-6, atol=1e-8)
+        x2 = (x64 * 0.5).float().double()
+        want2 = OL.join_straight(ora.forward(x2, w64))
+        tw2 = OL.join_straight(twin.forward(x2.float(), w64.float()))
+        out2 = mod(x2.float().to(dev), straight_output=True)
+        assert_close(out2, want2, "second step forward", tw2)
+        assert_close(mod.bnWMM.bn_stds, torch.from_numpy(ora.stds_flat()), "running stds step 2",
+                     torch.from_numpy(twin.stds_flat().astype(np.float64)), rtol=5e-6, atol=1e-8)
         # eval mode leaves the statistics alone
         mod.eval()
-        ora.training = False
+        ora.training = twin.training = False
         keep = mod.bnWMM.bn_stds.clone()
         out3 = mod(x.detach(), straight_output=False)
-        want3 = ora.forward(xo.detach(), wo.detach())
+        want3 = ora.forward(x64, w64)
+        tw3 = twin.forward(x64.float(), w64.float())
         assert torch.equal(keep, mod.bnWMM.bn_stds) and mod.bnWMM.bn_cnt == 3.0
-        for a, b in zip(out3, want3):
-            assert_close(a, b, "eval forward")
+        for a, b, c in zip(out3, want3, tw3):
+            assert_close(a, b, "eval forward", c)
+
+
+def test_layer_config5_shape(dev):
+    """One 16 -> 16 channel layer of benchmark configuration 5 (L=20, default triples), B=1, one training step:
+    the three-tile matrix-core backward, the two-class forward launch and the stream join that shape takes."""
+    lmax, tau = 20, [16] * 21
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tau, tau, False, True, seed=20)
+    x64 = rand_straight(tau, 1, seed=22)
+    go64 = randn32((1, 16 * 441, 2), torch.Generator().manual_seed(24))
+    check_layer_step(dev, mod, ora, twin, w64, x64, go64)
 
 
 def _random_layer_cases(n, seed, out_lo=1):
@@ -421,22 +501,12 @@ def _random_layer_cases(n, seed, out_lo=1):
 def test_layer_random_shapes(dev, lmax, tin, tout, bsz, sparse, bn, k):
     """Seeded random degrees, ragged channel counts (degrees without input or without output channels
     included), batch sizes and triple sets: one training step of the layer, forward and both gradients, against the oracle."""
-    mod, ora, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=100 + k)
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=100 + k)
     x64 = rand_straight(tin, bsz, seed=200 + k)
     g = torch.Generator().manual_seed(300 + k)
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
-    go64 = torch.randn(bsz, n_o, 2, generator=g, dtype=torch.float64)
-    xo = x64.float().double().requires_grad_(True)
-    wo = w64.clone().requires_grad_(True)
-    want = OL.join_straight(ora.forward(xo, wo))
-    want_gx, want_gw = torch.autograd.grad(want, (xo, wo), go64, allow_unused=True)
-    x = x64.float().to(dev).requires_grad_(True)
-    out = mod(x, straight_output=True)
-    assert_close(out, want, "layer forward")
-    out.backward(go64.float().to(dev))
-    assert_close(x.grad, want_gx if want_gx is not None else torch.zeros_like(xo), "layer grad F")
-    if wo.numel():
-        assert_close(mod.bnWMM.W.grad, want_gw, "layer grad W")
+    go64 = randn32((bsz, n_o, 2), g)
+    check_layer_step(dev, mod, ora, twin, w64, x64, go64)
 
 
 def test_layer_backward_two_streams_matches_one_stream(dev, monkeypatch):
@@ -451,7 +521,7 @@ def test_layer_backward_two_streams_matches_one_stream(dev, monkeypatch):
     results = []
     for overlap in (1, 0):
         monkeypatch.setattr(CG_layers, "_OVERLAP_GRAD_W", overlap)
-        mod, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=7)
+        mod, _, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=7)
         mod.train()
         xs = x.clone().requires_grad_(True)
         for go in gos:                                   # gradients accumulate over the steps
@@ -461,53 +531,83 @@ def test_layer_backward_two_streams_matches_one_stream(dev, monkeypatch):
         assert torch.equal(a, b)
 
 
-def test_spherical_cnn_stack(dev):
-    from cgnet_amd import CGNet
-    lmax = 4
-    taus = [[1] * 5, [3] * 5, [2, 3, 2, 1, 2]]
-    net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
-    assert net.output_length == 2 * (1 + 3 + 2)
-    layers, ws = [], []
-    g = torch.Generator().manual_seed(3)
-    for i, cg in enumerate(net.cgs):
-        ora = OL.LayerOracle(lmax, taus[i], taus[i + 1], cg.cg.lll_list, batchnorm=True)
-        t_ff = [int(v) for v in cg.t_FF]
-        w64 = torch.randn(sum(a * b for a, b in zip(t_ff, taus[i + 1])), 2, generator=g, dtype=torch.float64) * 0.3
-        stds = 0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
-        with torch.no_grad():
-            cg.bnWMM.W.copy_(w64.float())
-            cg.bnWMM.bn_stds.copy_(stds.float())
-        ora.set_stds_flat(stds.float().double().numpy())
-        layers.append(ora)
-        ws.append(w64.float().double().requires_grad_(True))
-    # real-signal symmetry f_l^{-m} = (-1)^m conj(f_l^m)
-    bsz = 3
+def real_signal_coefficients(lmax, bsz, gen):
+    """Straight (bsz, (lmax+1)^2, 2) coefficients of a real signal, one channel per degree:
+    f_l^{-m} = (-1)^m conj(f_l^m), f_l^0 real."""
     parts = []
     for l in range(lmax + 1):
-        z = torch.randn(bsz, 1, 2 * l + 1, 2, generator=g, dtype=torch.float64)
+        z = torch.randn(bsz, 1, 2 * l + 1, 2, generator=gen, dtype=torch.float64)
         for m in range(1, l + 1):
             sign = (-1.0) ** m
             z[:, :, l - m, 0] = sign * z[:, :, l + m, 0]
             z[:, :, l - m, 1] = -sign * z[:, :, l + m, 1]
         z[:, :, l, 1] = 0
         parts.append(z.reshape(bsz, -1, 2))
-    x64 = torch.cat(parts, 1).float().double()
-    xo = x64.clone().requires_grad_(True)
-    want = OL.stack_forward(layers, ws, xo, taus[0], skipconn=True)
-    head = torch.randn(want.shape[1], 10, generator=g, dtype=torch.float64) * 0.2
+    return torch.cat(parts, 1).float().double()
+
+
+def test_spherical_cnn_stack(dev):
+    from cgnet_amd import CGNet
+    lmax = 4
+    taus = [[1] * 5, [3] * 5, [2, 3, 2, 1, 2]]
+    net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
+    assert net.output_length == 2 * (1 + 3 + 2)
+    layers, twins, ws = [], [], []
+    g = torch.Generator().manual_seed(3)
+    for i, cg in enumerate(net.cgs):
+        t_ff = [int(v) for v in cg.t_FF]
+        w64 = (torch.randn(sum(a * b for a, b in zip(t_ff, taus[i + 1])), 2, generator=g, dtype=torch.float64) * 0.3).float().double()
+        stds = (0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)).float()
+        with torch.no_grad():
+            cg.bnWMM.W.copy_(w64.float())
+            cg.bnWMM.bn_stds.copy_(stds)
+        layers.append(make_oracle(lmax, taus[i], taus[i + 1], cg.cg.lll_list, True, stds))
+        twins.append(make_oracle(lmax, taus[i], taus[i + 1], cg.cg.lll_list, True, stds, dtype=F32))
+        ws.append(w64)
+    bsz = 3
+    x64 = real_signal_coefficients(lmax, bsz, g)
+    head = (torch.randn(net.output_length, 10, generator=g, dtype=torch.float64) * 0.2).float().double()
     labels = torch.randint(0, 10, (bsz,), generator=g)
-    loss_o = torch.nn.functional.cross_entropy(want @ head, labels)
-    grads_o = torch.autograd.grad(loss_o, [xo] + ws)
+
+    def run(oracles, dtype):
+        xo = x64.to(dtype).clone().requires_grad_(True)
+        wo = [w.to(dtype).clone().requires_grad_(True) for w in ws]
+        emb = OL.stack_forward(oracles, wo, xo, taus[0], skipconn=True)
+        loss = torch.nn.functional.cross_entropy(emb @ head.to(dtype), labels)
+        return emb.detach(), torch.autograd.grad(loss, [xo] + wo)
+    want, grads_o = run(layers, F64)
+    tw, grads_t = run(twins, F32)
 
     x = x64.float().to(dev).requires_grad_(True)
     emb = net(x)
     assert emb.shape == (bsz, net.output_length)
-    assert_close(emb, want, "stack embedding", rtol=2e-5, atol=2e-6)
-    loss = torch.nn.functional.cross_entropy(emb.double() @ head.to(dev), labels.to(dev))
+    assert_close(emb, want, "stack embedding", tw)
+    loss = torch.nn.functional.cross_entropy(emb @ head.float().to(dev), labels.to(dev))
     loss.backward()
-    assert_close(x.grad, grads_o[0], "stack grad input", rtol=1e-4, atol=2e-6)
+    assert_close(x.grad, grads_o[0], "stack grad input", grads_t[0])
     for i, cg in enumerate(net.cgs):
-        assert_close(cg.bnWMM.W.grad, grads_o[1 + i], "stack grad W%d" % i, rtol=1e-4, atol=2e-6)
+        assert_close(cg.bnWMM.W.grad, grads_o[1 + i], "stack grad W%d" % i, grads_t[1 + i])
+
+
+def test_spherical_cnn_fast_constructor(dev):
+    """The constructor the reference's Shrec17 script calls (Shrec17_main_fast.py:78-79): one tau list for all
+    layers, ``num_channels_input`` channels per degree on the way in, skip_type 1 / 0 = embedding with / without
+    skip connections.  Same layers as the equivalent SphericalCNN, hence the same numbers."""
+    from cgnet_amd import CGNet
+    lmax, taus, nlayers, cin, bsz = 3, [3, 2, 2, 1], 2, 6, 4
+    for skip in (1, 0):
+        torch.manual_seed(11); np.random.seed(11)
+        fast = CGNet.SphericalCNN_fast(lmax, taus, nlayers, skip_type=skip, num_channels_input=cin)
+        torch.manual_seed(11); np.random.seed(11)
+        slow = CGNet.SphericalCNN(lmax, [[cin] * (lmax + 1)] + [taus] * nlayers, skipconn=bool(skip))
+        assert fast.output_length == (2 * (cin + nlayers * taus[0]) if skip else 2 * taus[0])
+        assert list(fast.state_dict()) == list(slow.state_dict())
+        x = rand_straight([cin] * (lmax + 1), bsz, seed=2).float().to(dev)
+        out = fast(x)
+        assert out.shape == (bsz, fast.output_length)
+        assert torch.equal(out, slow(x))
+    with pytest.raises(NotImplementedError):
+        CGNet.SphericalCNN_fast(lmax, taus, nlayers, skip_type=2, num_channels_input=cin)
 
 
 # ------------------------------------------------------------------------------- full-size properties
@@ -569,6 +669,7 @@ def test_full_size_layer_config3_runs(dev):
     mod2.load_state_dict(mod.state_dict())
     with torch.no_grad():
         mod2.bnWMM.bn_stds.fill_(1.0)
+    mod2.bnWMM.bn_cnt = 1.0                               # the state dictionary carried the advanced count
     mod2.fused = False
     out2 = mod2(x.detach(), straight_output=True)
     assert torch.allclose(out, out2, rtol=1e-5, atol=1e-6)
@@ -589,7 +690,8 @@ def test_full_size_properties_config4(dev, sparse):
     assert torch.equal(y5[0], y[5])                                               # samples independent
     # against the oracle on one sample (the CPU restatement needs seconds for one sample of this size)
     want, _ = cg_oracle_fwd_bwd(lmax, taus, mod.lll_list, x[5:6].double().cpu())
-    assert_close(y5, want, "config 4 forward, one sample")
+    tw, _ = cg_oracle_fwd_bwd(lmax, taus, mod.lll_list, x[5:6].double().cpu(), dtype=F32)
+    assert_close(y5, want, "config 4 forward, one sample", tw)
     # adjoint identity of the bilinear map
     dx = 1e-2 * torch.randn_like(x)
     gy = torch.randn_like(y)
@@ -600,6 +702,10 @@ def test_full_size_properties_config4(dev, sparse):
     lhs = float((gy.double() * jdx).sum())
     rhs = float((xr.grad.double() * dx.double()).sum())
     assert lhs == pytest.approx(rhs, rel=2e-4)
+    # the gradient of one sample of the full batch against the oracle
+    _, want_g = cg_oracle_fwd_bwd(lmax, taus, mod.lll_list, x[5:6].double().cpu(), gy[5:6].double().cpu())
+    _, tw_g = cg_oracle_fwd_bwd(lmax, taus, mod.lll_list, x[5:6].double().cpu(), gy[5:6].double().cpu(), dtype=F32)
+    assert_close(xr.grad[5:6], want_g, "config 4 backward, one sample of the batch", tw_g)
 
 
 def test_full_size_stack_config5_runs(dev):
@@ -612,7 +718,7 @@ def test_full_size_stack_config5_runs(dev):
     net = CGNet.SphericalCNN(lmax, taus, norm=True, skipconn=True, sparse_flag=False)
     assert net.output_length == 2 * (1 + 4 * 16)
     g = torch.Generator().manual_seed(5)
-    x = rand_straight(taus[0], bsz, 5).float()
+    x = real_signal_coefficients(lmax, bsz, g).float()    # spherical-harmonic coefficients of a real signal
     head = torch.nn.Linear(net.output_length, 10).to(dev)
     labels = torch.randint(0, 10, (bsz,), generator=g).to(dev)
     x = x.to(dev).requires_grad_(True)
@@ -665,19 +771,20 @@ def test_classifier_from_coefficient_file(dev, tmp_path):
     # layer 0 alone against the oracle (injected weights and statistics)
     cg0 = net.SphericalCNN.cgs[0]
     taus_in, taus_out = [1] * n_deg, model.define_taus(2, 4, n_deg - 1)
-    ora = OL.LayerOracle(n_deg - 1, taus_in, taus_out, cg0.cg.lll_list, batchnorm=True)
     g = torch.Generator().manual_seed(0)
     t_ff = [int(v) for v in cg0.t_FF]
-    w64 = torch.randn(sum(a * b for a, b in zip(t_ff, taus_out)), 2, generator=g, dtype=torch.float64) * 0.3
-    stds = 0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)
+    w64 = (torch.randn(sum(a * b for a, b in zip(t_ff, taus_out)), 2, generator=g, dtype=torch.float64) * 0.3).float().double()
+    stds = (0.5 + torch.rand(sum(t_ff), generator=g, dtype=torch.float64)).float()
     with torch.no_grad():
         cg0.bnWMM.W.copy_(w64.float())
-        cg0.bnWMM.bn_stds.copy_(stds.float())
-    ora.set_stds_flat(stds.float().double().numpy())
-    ora.training = False
+        cg0.bnWMM.bn_stds.copy_(stds)
+    ora = make_oracle(n_deg - 1, taus_in, taus_out, cg0.cg.lll_list, True, stds)
+    twin = make_oracle(n_deg - 1, taus_in, taus_out, cg0.cg.lll_list, True, stds, dtype=F32)
+    ora.training = twin.training = False
     cg0.eval()
-    want = OL.join_straight(ora.forward(x.double().cpu(), w64.float().double()))
-    assert_close(cg0(x, straight_output=True), want, "first layer on file input")
+    want = OL.join_straight(ora.forward(x.double().cpu(), w64))
+    tw = OL.join_straight(twin.forward(x.cpu(), w64.float()))
+    assert_close(cg0(x, straight_output=True), want, "first layer on file input", tw)
     # the whole classifier
     net.train()
     logp = net(x)
@@ -691,7 +798,14 @@ def test_classifier_from_coefficient_file(dev, tmp_path):
     counts = CGNet.normalisation_counts(net)
     assert counts == {"SphericalCNN.cgs.0.bnWMM": 2.0, "SphericalCNN.cgs.1.bnWMM": 2.0}
     net2 = model.MNIST_Net(n_deg - 1, tau_type=2, tau_man=4, nlayers=2, dropout=None)
-    net2.load_state_dict(net.state_dict())
+    sd = net.state_dict()
+    assert float(sd["SphericalCNN.cgs.1.bnWMM.bn_cnt"]) == 2.0     # the count travels with the checkpoint
+    net2.load_state_dict(sd)
+    assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
+    # a checkpoint written by the reference has no such entry: it loads, and the helper restores the counts
+    net2.SphericalCNN.cgs[1].bnWMM.bn_cnt = 7.0
+    net2.load_state_dict({k: v for k, v in sd.items() if not k.endswith("bn_cnt")})
+    assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 7.0
     CGNet.load_normalisation_counts(net2, counts)
     assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
     net.eval(); net2.eval()

@@ -84,6 +84,16 @@ def test_mst_matches_scipy_fixture(golden_dir, lmax):
         assert list(zip(t1, t2)) == [p for p in want[l] if p[0] != p[1]]
 
 
+def test_mst_equals_scipy_live_for_every_degree_up_to_24():
+    """The product's own Kruskal against scipy's minimum_spanning_tree (the routine the reference calls,
+    CGutils.py:73-98) for EVERY lmax a user is likely to pick, not only the sizes in the fixture; ties included."""
+    pytest.importorskip("scipy")
+    for lmax in range(0, 25):
+        want = T.mst_pairs(lmax, use_scipy=True)
+        assert S.compute_mst_ltuples(lmax) == [[(int(a), int(b)) for a, b in per_l] for per_l in want], lmax
+        assert T.mst_pairs(lmax, use_scipy=False) == want, lmax
+
+
 @pytest.mark.parametrize("lmax,count", [(11, 229), (15, 417), (20, 731)])
 def test_mst_properties(lmax, count):
     pairs = T.mst_pairs(lmax, use_scipy=True)
