@@ -29,6 +29,8 @@ SIGNATURES = {
     "cgnet_sparse_forward": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp]),
     "cgnet_sparse_forward_stats_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_sparse_forward_stats": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_sparse_forward_stats_static_limit": (ctypes.c_size_t, []),
+    "cgnet_sparse_forward_stats_static": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp, _vp]),
     "cgnet_sparse_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_sparse_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "cgnet_wmm_plan_create": (ctypes.c_int, [ctypes.POINTER(_vp), ctypes.c_int, _c_int_p, _c_int_p]),

@@ -117,6 +117,19 @@ class CGPlan:
             _lib.check(lib.cgnet_sparse_forward_stats(self._h, _ptr(F), _ptr(FF), _ptr(CG), int(B), _ptr(sums),
                                                       _ptr(ws), ws.numel(), _stream(F.device)))
 
+    def forward_stats_static(self, F, FF, CG, B, sums):
+        """``forward_stats`` through the entry point that allocates nothing (partial sums in the
+        library's fixed area; raises when they do not fit)."""
+        self._check_io(F, B)
+        _require_gpu("output", FF)
+        _require_gpu("CG", CG)
+        _require_gpu("sums", sums, torch.float64)
+        if FF.numel() != B * self.nFF * 2 or sums.numel() != 2 * self.sum_tFF or CG.numel() < self.cg_len:
+            raise RuntimeError("forward_stats_static: tensor sizes do not match the plan")
+        with torch.cuda.device(F.device):
+            _lib.check(_lib.load().cgnet_sparse_forward_stats_static(self._h, _ptr(F), _ptr(FF), _ptr(CG), int(B),
+                                                                     _ptr(sums), _stream(F.device)))
+
     def backward(self, F, gF, gFF, CG, B):
         self._check_io(F, B)
         _require_gpu("grad_in", gF)

@@ -20,6 +20,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -1210,7 +1211,41 @@ partial_sum_kernel(const float2* __restrict__ part, float2* __restrict__ out, si
     out[i] = s;
 }
 
+__global__ void __launch_bounds__(256) fill_zero_f64_kernel(double* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.;
+}
+
 // ------------------------------------------------------------------------------------- host
+// Partial statistics of cgnet_sparse_forward_stats_static: a fixed area every GPU the library runs
+// on holds until the process ends.  In host code the array's name is only a handle; its device
+// address is resolved once per device (resolve_static_scratch) and that pointer is what kernels get.
+constexpr size_t kStaticScratchBytes = 16u << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (nullptr and an error message on failure).
+void* resolve_static_scratch() {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        set_error("cannot identify the current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_error("hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[device] = ptr;
+    }
+    return g_scratch_ptr[device];
+}
+
 int samples_per_group_for(int B, int ntasks) {
     // enough work-groups to fill 256 CUs a few times over, while each group amortises the
     // staging of its CG table over several samples
@@ -1699,6 +1734,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     }
 
     CGNET_HIP(hipGetDevice(&p->device));
+    // set-up time: the statistics area of cgnet_sparse_forward_stats_static gets its address on this device
+    CGNET_REQUIRE(resolve_static_scratch() != nullptr, CGNET_ERR_HIP, "%s", cgnet_last_error());
     if (!p->fwd_tasks.empty()) {
         CGNET_HIP(hipMalloc((void**)&p->d_fwd_tasks, sizeof(CgTask) * p->fwd_tasks.size()));
         CGNET_HIP(hipMemcpy(p->d_fwd_tasks, p->fwd_tasks.data(), sizeof(CgTask) * p->fwd_tasks.size(), hipMemcpyHostToDevice));
@@ -1815,6 +1852,41 @@ extern "C" int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float
     const int n2 = 2 * plan->sumT;
     CGNET_LAUNCH(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
                        (const double*)d_workspace, d_sums, n2, ngroups);
+    CGNET_HIP(hipGetLastError());
+    return CGNET_OK;
+}
+
+extern "C" size_t cgnet_sparse_forward_stats_static_limit(void) { return kStaticScratchBytes; }
+
+extern "C" int cgnet_sparse_forward_stats_static(const cgnet_cg_plan* plan, const float* d_F, float* d_FF,
+                                                 const float* d_CG, int B, double* d_sums, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    if (plan->sumT == 0) return CGNET_OK;
+    CGNET_REQUIRE(d_sums, CGNET_ERR_ARG, "d_sums is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    const int n2 = 2 * plan->sumT;
+    if (B == 0 || plan->nFF == 0) {
+        // a fill kernel, not a memset: the call may be recorded into a graph
+        CGNET_LAUNCH(fill_zero_f64_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s, d_sums, n2);
+        CGNET_HIP(hipGetLastError());
+        return CGNET_OK;
+    }
+    CGNET_REQUIRE(d_F && d_FF && d_CG, CGNET_ERR_ARG, "null device pointer");
+    const size_t need = cgnet_sparse_forward_stats_workspace(plan, B);
+    CGNET_REQUIRE(need <= kStaticScratchBytes, CGNET_ERR_UNSUPPORTED,
+                  "the partial statistics of this call need %zu bytes, the static area holds %zu "
+                  "(use cgnet_sparse_forward_stats with a caller workspace)", need, kStaticScratchBytes);
+    void* area = resolve_static_scratch();   // resolved when the plan was created on this device; a lookup here
+    CGNET_REQUIRE(area, CGNET_ERR_HIP, "%s", cgnet_last_error());
+    const int spg = samples_per_group_for(B, (int)plan->fwd_tasks.size());
+    const int ngroups = (B + spg - 1) / spg;
+    // every partial sum [group][channel][2] of this call is written by the product kernel before the
+    // reduction reads it, so what an earlier call left in the area needs no clearing
+    int rc = launch_forward(plan, d_F, d_FF, d_CG, B, (double*)area, spg, s);
+    if (rc != CGNET_OK) return rc;
+    CGNET_LAUNCH(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s, (const double*)area, d_sums, n2, ngroups);
     CGNET_HIP(hipGetLastError());
     return CGNET_OK;
 }

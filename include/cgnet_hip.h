@@ -99,6 +99,18 @@ int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float* d_F, floa
                                const float* d_CG, int B, double* d_sums,
                                void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* cgnet_sparse_forward_stats for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same product and the same sums,
+ * bit for bit, but the partial sums live in a fixed area of cgnet_sparse_forward_stats_static_limit()
+ * bytes (16 MiB) inside the library instead of a caller workspace, and the call allocates nothing.
+ * It has no counterpart in the reference.  A call whose partial sums need more (16 * sum_l t_FF[l] *
+ * sample groups bytes, i.e. cgnet_sparse_forward_stats_workspace) returns CGNET_ERR_UNSUPPORTED.
+ * All calls on one GPU share that area: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe. */
+size_t cgnet_sparse_forward_stats_static_limit(void);
+int cgnet_sparse_forward_stats_static(const cgnet_cg_plan* plan, const float* d_F, float* d_FF,
+                                      const float* d_CG, int B, double* d_sums, void* stream);
+
 /* Gradient of the product with respect to F given d_gFF = dLoss/dFF:
  *   gF[b,l1,t1,m1] = sum CG * gFF[b,l,t,m1+m2] * conj(F[b,l2,t2,m2])  + the same with the
  *   roles of the two slots exchanged (a diagonal triple l1 == l2 contributes through both).
