@@ -17,6 +17,7 @@ import torch
 from torch import nn
 
 from . import CG_cuda_ops, CGutils, _lib
+from . import _plans
 from ._plans import CGPlan, WMMPlan
 
 BN_FLAG = _lib.FN_BATCHNORM
@@ -330,6 +331,7 @@ class CG_woFilter_cuda(nn.Module):
 
 # --------------------------------------------------------------------------- the whole layer
 _OVERLAP_GRAD_W = int(os.environ.get("CGNET_OVERLAP_GW", "1"))
+_FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "0")))
 _CU_LDS_BYTES = 160 * 1024
 _side_streams = {}
 
@@ -347,7 +349,8 @@ class _CGBN_fused(torch.autograd.Function):
     per-channel statistics come out of the product kernel instead of a second pass over FF."""
 
     @staticmethod
-    def forward(ctx, Fs, W, cg_plan, wmm_plan, CG, bn_stds, bn_cnt, bn_eps, training):
+    def forward(ctx, Fs, W, cg_plan, wmm_plan, CG, bn_stds, bn_cnt, bn_eps, training, fused_backward=False):
+        ctx.fused_backward = bool(fused_backward)
         Fs = Fs.contiguous()
         W = W.contiguous()
         B = Fs.shape[0]
@@ -372,9 +375,27 @@ class _CGBN_fused(torch.autograd.Function):
         Fs, W, FF, CG, stds = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         need_F, need_W = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        grad_FF = torch.empty_like(FF) if need_F else None
         grad_W = torch.empty_like(W) if need_W else None
         grad_F = None
+        if need_F and ctx.fused_backward and _plans.fused_backward_supported(ctx.cg_plan, ctx.wmm_plan):
+            # The gradient with respect to FF never exists in memory: the product's backward forms every
+            # tile of it in LDS from grad_output and the weights.  The weight gradient (which needs FF, not
+            # gFF) runs beside it on the second stream.
+            main = torch.cuda.current_stream(Fs.device)
+            overlap = need_W and _OVERLAP_GRAD_W
+            if need_W:
+                side = _side_stream(Fs.device) if overlap else main
+                if overlap:
+                    side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
+            grad_F = torch.empty_like(Fs)
+            _plans.fused_backward(ctx.cg_plan, ctx.wmm_plan, Fs, grad_F, grad_output, W, CG, ctx.B, stds, ctx.eps,
+                                  ctx.flags)
+            if overlap:
+                main.wait_stream(side)
+            return grad_F, grad_W, None, None, None, None, None, None, None, None
+        grad_FF = torch.empty_like(FF) if need_F else None
         if need_F and need_W and _OVERLAP_GRAD_W:
             # The weight gradient depends on nothing the other chain produces: it runs on a second
             # stream (default priority) beside grad FF.  Its tail may run into the CG backward only
@@ -393,13 +414,13 @@ class _CGBN_fused(torch.autograd.Function):
                 main.wait_stream(side)
             ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
             main.wait_stream(side)
-            return grad_F, grad_W, None, None, None, None, None, None, None
+            return grad_F, grad_W, None, None, None, None, None, None, None, None
         if need_F or need_W:
             ctx.wmm_plan.backward(grad_output, grad_FF, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
         if need_F:
             grad_F = torch.empty_like(Fs)
             ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
-        return grad_F, grad_W, None, None, None, None, None, None, None
+        return grad_F, grad_W, None, None, None, None, None, None, None, None
 
 
 class CGBN_cuda(nn.Module):
@@ -416,6 +437,11 @@ class CGBN_cuda(nn.Module):
         self.tau_out = tau_out
         self.bnWMM = MyBatchNormWeightMM_cuda(lmax, self.t_FF, tau_out, batchnorm, weight_scale, init, eps, device)
         self.fused = True      # False: chain the two reference Functions (separate statistics pass)
+        # With ``fused``: True takes the backward from grad_output to the input gradient in one kernel, without a
+        # grad_FF tensor (B x nFF complex) in memory, where the shapes allow it
+        # (cgnet_CGBN_backward_fused_supported); same gradients, bit for bit.  Off by default: at the benchmark
+        # shape it saves the memory but no time yet (CGNET_FUSED_BACKWARD=1 turns it on for new layers).
+        self.fused_backward = _FUSED_BACKWARD
         self.to(device)
 
     def forward(self, fs, straight_output=False):
@@ -427,7 +453,7 @@ class CGBN_cuda(nn.Module):
             assert fs.is_cuda
             bn = self.bnWMM
             new_fs = _CGBN_fused.apply(fs, bn.W, self.cg.native_plan(), bn.native_plan(), self.cg.CGspace,
-                                       bn.bn_stds, bn.bn_cnt, bn._eps_host, bn.training)
+                                       bn.bn_stds, bn.bn_cnt, bn._eps_host, bn.training, self.fused_backward)
             if bn.batchnorm and bn.training:
                 bn.bn_cnt += 1
         else:

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libcgnet_hip.so")
+# CGNET_HIP_LIBRARY names another build of the same library (kernel experiments); the default is the in-tree one
+LIB_PATH = os.environ.get("CGNET_HIP_LIBRARY") or os.path.join(_HERE, "csrc", "libcgnet_hip.so")
 
 OK, ERR_ARG, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED = 0, -1, -2, -3, -4
 FN_BATCHNORM, FN_UPDATE_STD = 0x1, 0x2
@@ -42,6 +43,10 @@ SIGNATURES = {
     "cgnet_FN_WMM_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_FN_WMM_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                              ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_CGBN_backward_fused_supported": (ctypes.c_int, [_vp, _vp]),
+    "cgnet_CGBN_backward_fused_workspace": (ctypes.c_size_t, [_vp, _vp, ctypes.c_int]),
+    "cgnet_CGBN_backward_fused": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
+                                                 ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_wmm_plan_gradw_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_profile_enable": (ctypes.c_int, [ctypes.c_int]),

@@ -215,3 +215,30 @@ class WMMPlan:
             _lib.check(lib.cgnet_FN_WMM_backward(self._h, _ptr(gO), _ptr(gFF), _ptr(gW), _ptr(FF), _ptr(W), int(B),
                                                  _ptr(stds), float(eps), int(flags), _ptr(ws), ws.numel(),
                                                  _stream(FF.device)))
+
+
+def fused_backward_supported(cg_plan, wmm_plan):
+    """Whether ``fused_backward`` takes this pair of plans (see cgnet_CGBN_backward_fused_supported)."""
+    return bool(_lib.load().cgnet_CGBN_backward_fused_supported(cg_plan._h, wmm_plan._h))
+
+
+def fused_backward(cg_plan, wmm_plan, F, gF, gO, W, CG, B, stds, eps, flags):
+    """gF of the whole layer straight from gO (no gFF in memory): cgnet_CGBN_backward_fused."""
+    _require_gpu("input", F)
+    _require_gpu("grad_in", gF)
+    _require_gpu("grad_out", gO)
+    _require_gpu("W", W)
+    _require_gpu("CG", CG)
+    if flags & _lib.FN_BATCHNORM:
+        _require_gpu("FN_stds", stds)
+    else:
+        stds = None
+    if (F.numel() != B * cg_plan.nF * 2 or gF.numel() != F.numel() or gO.numel() != B * wmm_plan.nO * 2
+            or W.numel() != wmm_plan.nW * 2 or CG.numel() < cg_plan.cg_len):
+        raise RuntimeError("fused backward: tensor sizes do not match the plans")
+    lib = _lib.load()
+    with torch.cuda.device(F.device):
+        ws = _workspace(lib.cgnet_CGBN_backward_fused_workspace(cg_plan._h, wmm_plan._h, int(B)), F.device)
+        _lib.check(lib.cgnet_CGBN_backward_fused(cg_plan._h, wmm_plan._h, _ptr(F), _ptr(gF), _ptr(gO), _ptr(W), _ptr(CG),
+                                                 int(B), _ptr(stds), float(eps), int(flags), _ptr(ws), ws.numel(),
+                                                 _stream(F.device)))

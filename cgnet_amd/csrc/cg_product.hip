@@ -65,6 +65,29 @@ struct BwdUTask {
     int TI, RW;               // slot-2 tiling for this run of equal l2
 };
 
+// Fused layer backward, packing kernels: what packing a task's weights needs to know (one entry per BwdUTask).
+struct GenTask {
+    int aoff;                 // float offset of the task's block in the packed conj(W)/div operand
+    int nks;                  // k-steps of 4 over (output channel, re/im); 0 for a degree without output channels
+    int tO;                   // output channels of degree l
+    int chan0, nch;           // the tile's channels inside degree l: first, count (rows * tau2)
+    int cumW, K, cumT;        // degree l: complex offset of its weights, mid channels, first mid channel among all
+};
+
+// Fused layer backward, main kernel: everything a stage needs to know of its task, 12 ints that a wave reads
+// with scalar loads one stage ahead.
+struct FusedTask {
+    int geom;                 // l | l2 << 8 | tau2 << 16 | first_of_l2 << 24 | last_of_l2 << 25
+    int offF2p;               // complex offset of degree l2 inside a sample's padded fragments
+    int cgp_off, cgp_len;     // the triple's zero-padded table (floats)
+    int p2off;                // complex offset of the (unit, l2) slab in a sample's slot-2 partial area
+    int aoff;                 // float offset of the task's packed A operand
+    int shape;                // nks | tO << 8 | nch << 16
+    int boff;                 // float offset inside a sample's packed B operand of degree l
+    int chunks;               // 16-byte pieces: A block | B block << 16
+    int pad[3];
+};
+
 }  // namespace cgnet
 
 struct cgnet_cg_plan {
@@ -96,6 +119,18 @@ struct cgnet_cg_plan {
     int bwd_P2 = 0;                              // complex entries of one sample's slot-2 partial area
     size_t bwd_fast_lds = 0;
     int device = 0;
+    // fused layer backward: per-task metadata for the mixing plan this plan was linked with last (rebuilt when the
+    // signature -- t_O and the offsets per degree -- changes)
+    mutable std::mutex fused_mu;
+    mutable std::vector<int> fused_signature;
+    mutable cgnet::GenTask* d_gens = nullptr;
+    mutable cgnet::FusedTask* d_ftasks = nullptr;
+    mutable int* d_packmap = nullptr;            // per block of the weight-packing kernel: (task, row tile)
+    mutable int* d_bmap = nullptr;               // per block of the gO-packing kernel: cumO, M, t_O, column tile | k-step << 8
+    mutable int fused_npack = 0, fused_nbmap = 0;
+    mutable size_t fused_operand_floats = 0;     // packed A operand, all tasks
+    mutable int fused_bop_floats = 0;            // packed B operand of one sample
+    mutable int fused_bcap = 0, fused_acap = 0;  // LDS bytes of the B / A operand buffers
 };
 
 namespace cgnet {
@@ -847,7 +882,9 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         const float2 *g, *f2;
         bwd_stage<NT>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+#ifndef CGNET_TEST_NOSLOT1
         bwd_accum<1, TI, RW>(q, cgp, g, f2, c.rtid, ax, ay);
+#endif
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
 #pragma unroll
@@ -1077,12 +1114,14 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
     if (cur.l2 <= 7) { CGNET_MM_NT(NK_, 1) }                            \
     else if (cur.l2 <= 15) { CGNET_MM_NT(NK_, 2) }                      \
     else { CGNET_MM_NT(NK_, 3) }
+#ifndef CGNET_TEST_NOSLOT2
         switch ((u.rows + 3) >> 2) {
             case 1: CGNET_MM(1) break;
             case 2: CGNET_MM(2) break;
             case 3: CGNET_MM(3) break;
             default: CGNET_MM(4) break;
         }
+#endif
 #undef CGNET_MM_NT
 #undef CGNET_MM_CALL
 #undef CGNET_MM
@@ -1139,6 +1178,328 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
     } else {
         bwd_hybrid_loop_b(c, u, t0, wave - u.nA, kHybWaves - u.nA, tid & 63, part2 + (size_t)b * P2);
     }
+}
+
+// ---- the layer's backward in one kernel: gFF tiles made in LDS ------------------------------------
+// cg_backward_hybrid_kernel whose work-groups make every task's gFF tile themselves instead of copying it from
+// memory:   gFF[c, (m, re/im)] = sum_k A[c][k] B[k][(m, re/im)],  k = (output channel to, re/im),
+//   A[c][(to,0)] = W_re[to][c]/div[c], A[c][(to,1)] = W_im[to][c]/div[c]
+//   B[(to,0)][(m,0)] = gO_re, B[(to,1)][(m,0)] = gO_im, B[(to,0)][(m,1)] = gO_im, B[(to,1)][(m,1)] = -gO_re
+// the arithmetic of wmm_gradff_mfma_kernel, instruction for instruction, so the tile holds the values that kernel
+// would have written to memory and the result equals the two-kernel route bit for bit.
+//
+// Both operands are packed beforehand in the order the lanes of a wave read them (pack_w_gen_kernel: one block per
+// task; pack_go_gen_kernel: one block per sample and degree), so that making the tile costs LDS reads and
+// matrix instructions but next to no vector-ALU work, which is what the kernel is short of.
+//
+// A stage (one task) has two phases.  Phase 1: all eight waves make the tile -- it is cut into units of 16 channels
+// x 16 real columns (one accumulator each), numbered column-tile major, and every wave takes a contiguous share.
+// Phase 2: the tile is used exactly as in the hybrid kernel (slot 1 on the vector ALUs, slot 2 on the matrix
+// cores).  The two operands of the next task's tile are copied into LDS during phase 2 (their buffers are only read
+// in phase 1), its coefficient table and l2 slab during the whole stage (double-buffered).  A wave learns about the
+// task after the next one through scalar loads that are in flight for a whole stage.
+__device__ __forceinline__ void lds_barrier() {      // this wave's LDS accesses are complete, then the group's barrier
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+struct FusedCtx {
+    const float2* Fp;          // this sample's fragments, rows padded with one zero
+    const float* Bg;           // this sample's packed B operand
+    const float* Ag;           // packed A operand, one block per task
+    const float* CGP;          // zero-padded tables of all triples
+    float2* f1;                // LDS: rows x (M1+1) slab of degree l1
+    char* f2;                  // LDS: two slabs of degree l2, f2cap bytes each
+    char* cg;                  // LDS: two tables, cgcap bytes each
+    float* bl;                 // LDS: the task's B operand
+    float* al;                 // LDS: the task's A operand
+    float* tile;               // LDS: the gFF tile
+    int f2cap, cgcap;
+    int tid, lane, wave;
+};
+
+__device__ __forceinline__ int ft_l(const FusedTask& t) { return t.geom & 255; }
+__device__ __forceinline__ int ft_l2(const FusedTask& t) { return (t.geom >> 8) & 255; }
+__device__ __forceinline__ int ft_tau2(const FusedTask& t) { return (t.geom >> 16) & 255; }
+__device__ __forceinline__ bool ft_first(const FusedTask& t) { return (t.geom >> 24) & 1; }
+__device__ __forceinline__ bool ft_last(const FusedTask& t) { return (t.geom >> 25) & 1; }
+__device__ __forceinline__ int ft_nks(const FusedTask& t) { return t.shape & 255; }
+__device__ __forceinline__ int ft_nch(const FusedTask& t) { return t.shape >> 16; }
+
+// Phase 1 of a stage: this wave's share of the tile.  al: the A operand, k-steps in pairs: float2 entry
+// [(row tile * NKP + kp) * 64 + lane] = (A of k-step 2kp, A of k-step 2kp+1), NKP = (NKS+1)/2, so that the 64 lanes of
+// a read touch 512 contiguous bytes; bl: entry [(column tile * NKS + ks) * 64 + lane].  Columns past 2M and rows
+// past the last channel are not stored.
+template <int NKS>
+__device__ __forceinline__ void gen_phase_nks(int nch, int M, const float* __restrict__ al, const float* __restrict__ bl,
+                                              float* __restrict__ tile, int wave, int lane) {
+    constexpr int NKP = (NKS + 1) / 2;
+    const int i = lane & 15, kk = lane >> 4;
+    const int M2f = 2 * M;
+    const int nct = (M2f + 15) >> 4, nrt = (nch + 15) >> 4, U = nct * nrt;
+    int idx = (wave * U) >> 3;
+    const int ue = ((wave + 1) * U) >> 3;
+    if (idx >= ue) return;
+    int ct = idx / nrt, rt = idx - ct * nrt;
+    while (idx < ue) {
+        const float* bp = bl + ct * (NKS * 64) + lane;
+        float bv[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) bv[ks] = bp[64 * ks];
+        const int col = 16 * ct + i;
+        const bool colok = col < M2f;
+        const int rt_end = min(nrt, rt + (ue - idx));
+        idx += rt_end - rt;
+        for (; rt < rt_end; ++rt) {
+            const float2* ap = reinterpret_cast<const float2*>(al) + rt * (NKP * 64) + lane;
+            float a[2 * NKP];
+#pragma unroll
+            for (int kp = 0; kp < NKP; ++kp) {
+                const float2 v = ap[64 * kp];
+                a[2 * kp] = v.x;
+                a[2 * kp + 1] = v.y;
+            }
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) acc = mfma4(a[ks], bv[ks], acc);
+            mfma_drain();
+            const int row = 16 * rt + 4 * kk;
+            float* dst = tile + row * M2f + col;
+            if (16 * rt + 16 <= nch) {               // wave-uniform: a full row tile
+                if (colok) {
+                    dst[0] = acc[0];
+                    dst[M2f] = acc[1];
+                    dst[2 * M2f] = acc[2];
+                    dst[3 * M2f] = acc[3];
+                }
+            } else if (colok) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (row + v < nch) dst[v * M2f] = acc[v];
+            }
+        }
+        rt = 0;
+        ++ct;
+    }
+}
+
+__device__ __forceinline__ void gen_phase(const FusedTask& t, const float* __restrict__ al, const float* __restrict__ bl,
+                                          float* __restrict__ tile, int wave, int lane) {
+    const int nch = ft_nch(t), M = 2 * ft_l(t) + 1;
+    switch (ft_nks(t)) {
+        case 0:      // a degree without output channels: its product channels have no gradient
+            for (int e = wave * 64 + lane; e < nch * 2 * M; e += kHybThreads) tile[e] = 0.f;
+            break;
+        case 1: gen_phase_nks<1>(nch, M, al, bl, tile, wave, lane); break;
+        case 2: gen_phase_nks<2>(nch, M, al, bl, tile, wave, lane); break;
+        case 3: gen_phase_nks<3>(nch, M, al, bl, tile, wave, lane); break;
+        case 4: gen_phase_nks<4>(nch, M, al, bl, tile, wave, lane); break;
+        case 5: gen_phase_nks<5>(nch, M, al, bl, tile, wave, lane); break;
+        case 6: gen_phase_nks<6>(nch, M, al, bl, tile, wave, lane); break;
+        case 7: gen_phase_nks<7>(nch, M, al, bl, tile, wave, lane); break;
+        default: gen_phase_nks<8>(nch, M, al, bl, tile, wave, lane); break;
+    }
+}
+
+// The loop over a unit's tasks, common to both roles; `work(task, table, l2 slab)` is phase 2.
+//   carried: cur = task k, nxt = task k+1 (both in scalar registers), loaded one stage before they are needed
+template <typename Work>
+__device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTask* __restrict__ ft, int ntask, Work work) {
+    FusedTask cur = ft[0];
+    FusedTask nxt = ft[min(1, ntask - 1)];
+    int f2par = 0;
+    for (int k = 0; k < ntask; ++k) {
+        dma_wait();
+        __syncthreads();       // everything copied for this stage has landed; nobody uses the tile or the other buffers
+        const FusedTask nxt2 = ft[min(k + 2, ntask - 1)];        // needed at the next stage
+        const bool more = k + 1 < ntask;
+        const int b = k & 1;
+        if (more) {
+            dma16<kHybThreads>(c.CGP + nxt.cgp_off, c.cg + (b ^ 1) * c.cgcap, nxt.cgp_len >> 2, c.tid);
+            if (ft_first(nxt))
+                dma16<kHybThreads>(c.Fp + nxt.offF2p, c.f2 + (f2par ^ 1) * c.f2cap,
+                                   (ft_tau2(nxt) * (2 * ft_l2(nxt) + 2)) >> 1, c.tid);
+        }
+#ifndef CGNET_TEST_NOGEN
+        gen_phase(cur, c.al, c.bl, c.tile, c.wave, c.lane);
+#endif
+#ifndef CGNET_TEST_NOBAR2
+        lds_barrier();         // the tile is complete; the operand buffers are free
+#endif
+        if (more) {
+            dma16<kHybThreads>(c.Ag + nxt.aoff, c.al, nxt.chunks & 0xffff, c.tid);
+            dma16<kHybThreads>(c.Bg + nxt.boff, c.bl, nxt.chunks >> 16, c.tid);
+        }
+        work(cur, reinterpret_cast<const float*>(c.cg + b * c.cgcap), reinterpret_cast<const float2*>(c.f2 + f2par * c.f2cap));
+        if (more && ft_first(nxt)) f2par ^= 1;
+        cur = nxt;
+        nxt = nxt2;
+    }
+}
+
+// Waves of role A (slot 1 on the vector ALUs), as bwd_unit_loop_a.
+template <int TI, int RW>
+__device__ __forceinline__ void fused_loop_a(const FusedCtx& c, const BwdUnit& u, const FusedTask* __restrict__ ft,
+                                             float2* __restrict__ dst) {
+    float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
+#pragma unroll
+    for (int i = 0; i < kBwdMaxTI; ++i) {
+        ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
+        tx[i][0] = tx[i][1] = ty[i][0] = ty[i][1] = 0.f;
+    }
+    fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
+        const BwdGeom q{ft_l(t), u.l1, ft_l2(t), u.rows, ft_tau2(t)};
+        bwd_accum<1, TI, RW>(q, cgp, reinterpret_cast<const float2*>(c.tile), f2, c.tid, ax, ay);
+        if (ft_last(t)) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    tx[i][j] += ax[i][j];
+                    ty[i][j] += ay[i][j];
+                    ax[i][j] = ay[i][j] = 0.f;
+                }
+        }
+    });
+    bwd_flush<TI, RW>(u.rows, 2 * u.l1 + 1, c.tid, tx, ty, dst);
+}
+
+// Matrix-core waves (slot 2), as bwd_hybrid_loop_b.
+__device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u, const FusedTask* __restrict__ ft,
+                                             int part, int split, float2* __restrict__ part2_b) {
+    f32x4 dre[kHybMaxTiles], dim[kHybMaxTiles];
+#pragma unroll
+    for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
+        const int l2 = ft_l2(t), tau2 = ft_tau2(t);
+        const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2};
+        const float2* g = reinterpret_cast<const float2*>(c.tile);
+#define CGNET_MM_CALL(NK_, NT_, KF_) bwd_mm_task<NK_, NT_, KF_>(q, cgp, g, c.f1, part, split, c.lane, dre, dim)
+#define CGNET_MM_NT(NK_, NT_)                                           \
+    if (u.rows & 3) CGNET_MM_CALL(NK_, NT_, false);                     \
+    else CGNET_MM_CALL(NK_, NT_, true);
+#define CGNET_MM(NK_)                                                   \
+    if (l2 <= 7) { CGNET_MM_NT(NK_, 1) }                                \
+    else if (l2 <= 15) { CGNET_MM_NT(NK_, 2) }                          \
+    else { CGNET_MM_NT(NK_, 3) }
+        switch ((u.rows + 3) >> 2) {
+            case 1: CGNET_MM(1) break;
+            case 2: CGNET_MM(2) break;
+            case 3: CGNET_MM(3) break;
+            default: CGNET_MM(4) break;
+        }
+#undef CGNET_MM_NT
+#undef CGNET_MM_CALL
+#undef CGNET_MM
+        if (ft_last(t)) {
+            const int M2 = 2 * l2 + 1;
+            mfma_drain();
+            bwd_mm_store(dre, dim, tau2, M2, c.lane, part2_b + t.p2off + (size_t)part * tau2 * M2);
+#pragma unroll
+            for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+    });
+}
+
+// LDS map (bytes): [16 zero] f1 | f2 x2 | table x2 | B operand | A operand | [16 zero] tile [16 zero]
+__host__ __device__ inline size_t bwd_fused_lds(int f1cap, int f2cap, int cgcap, int tcap, int bcap, int acap) {
+    return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + (size_t)bcap + (size_t)acap + 16 + (size_t)tcap + 16;
+}
+
+__global__ void __launch_bounds__(kHybThreads, 4)
+cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restrict__ Bg, const float* __restrict__ Ag,
+                           const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
+                           const BwdUnit* __restrict__ units, const FusedTask* __restrict__ ftasks, int nF, int nFp,
+                           int nBg, int P2, int f1cap, int f2cap, int cgcap, int tcap, int bcap, int acap, int B) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const UnitPart up = unit_major(B);
+    const BwdUnit u = units[up.unit];
+    const int b = up.part;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M1 = 2 * u.l1 + 1;
+    const bool roleA = wave < u.nA;                  // wave-uniform
+    FusedCtx c;
+    c.Fp = Fp + (size_t)b * nFp;
+    c.Bg = Bg + (size_t)b * nBg;
+    c.Ag = Ag;
+    c.CGP = CGP;
+    c.f1 = reinterpret_cast<float2*>(smem + 16);
+    c.f2 = reinterpret_cast<char*>(smem) + 16 + f1cap;
+    c.cg = c.f2 + 2 * f2cap;
+    c.bl = reinterpret_cast<float*>(c.cg + 2 * cgcap);
+    c.al = reinterpret_cast<float*>(reinterpret_cast<char*>(c.bl) + bcap);
+    c.tile = reinterpret_cast<float*>(reinterpret_cast<char*>(c.al) + acap + 16);
+    c.f2cap = f2cap; c.cgcap = cgcap;
+    c.tid = tid; c.lane = tid & 63; c.wave = wave;
+    {
+        const int n16 = (int)(bwd_fused_lds(f1cap, f2cap, cgcap, tcap, bcap, acap) >> 4);
+        float4* z = reinterpret_cast<float4*>(smem);
+        for (int e = tid; e < n16; e += kHybThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __syncthreads();                                 // the clearing stores precede every copy
+    const FusedTask* ft = ftasks + u.task_begin;
+    const FusedTask t0 = ft[0];
+    dma16<kHybThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
+    dma16<kHybThreads>(c.CGP + t0.cgp_off, c.cg, t0.cgp_len >> 2, tid);
+    dma16<kHybThreads>(c.Fp + t0.offF2p, c.f2, (ft_tau2(t0) * (2 * ft_l2(t0) + 2)) >> 1, tid);
+    dma16<kHybThreads>(c.Ag + t0.aoff, c.al, t0.chunks & 0xffff, tid);
+    dma16<kHybThreads>(c.Bg + t0.boff, c.bl, t0.chunks >> 16, tid);
+    // the first stage waits for these copies
+    if (roleA) {
+        float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
+#define CGNET_LOOP_A(TI_, RW_) fused_loop_a<TI_, RW_>(c, u, ft, dst)
+        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#undef CGNET_LOOP_A
+    } else {
+        fused_loop_b(c, u, ft, wave - u.nA, kHybWaves - u.nA, part2 + (size_t)b * P2);
+    }
+}
+
+// The A operand of the fused kernel, one block per task, k-steps in pairs (nkp = (nks+1)/2 pairs, an odd last one
+// padded with zeros): float2 entry [(row tile * nkp + kp) * 64 + lane] = (A[c][4(2kp) + kk], A[c][4(2kp+1) + kk]) for
+// c = chan0 + 16 * row tile + lane % 16, kk = lane / 16; rows past the tile's last channel and k past 2 t_O are
+// zero.  One work-group of 64 threads per (task, row tile).
+__global__ void __launch_bounds__(64)
+pack_w_gen_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                  const GenTask* __restrict__ gens, const int* __restrict__ map, float* __restrict__ Ag) {
+    const GenTask g = gens[map[2 * blockIdx.x]];
+    const int rt = map[2 * blockIdx.x + 1];
+    const int lane = threadIdx.x, i = lane & 15, kk = lane >> 4;
+    const int cl = 16 * rt + i;
+    const bool on = cl < g.nch;
+    const int c = g.chan0 + cl;
+    const int nkp = (g.nks + 1) >> 1;
+    float* dst = Ag + g.aoff + ((size_t)rt * nkp * 64 + lane) * 2;       // float2 entry [(rt * nkp + kp) * 64 + lane]
+    const float r = (on && stds) ? fmaxf(eps, stds[g.cumT + c]) : 1.f;
+    for (int ks = 0; ks < 2 * nkp; ++ks) {
+        const int k = 4 * ks + kk, to = k >> 1;
+        float v = 0.f;
+        if (on && ks < g.nks && to < g.tO) {
+            const float2 w = W[g.cumW + (size_t)to * g.K + c];
+            v = (k & 1) ? w.y : w.x;
+            if (stds) v = v / r;
+        }
+        dst[(size_t)(ks >> 1) * 128 + (ks & 1)] = v;
+    }
+}
+
+// The B operand of the fused kernel, per sample and degree: entry [(column tile * nks + ks) * 64 + lane] =
+// B[k][col] for k = 4 * ks + lane / 16 = (to, re/im), col = 16 * column tile + lane % 16 = (m, re/im); k past 2 t_O
+// and columns past 2M are zero.  map: per block (cumO, M, t_O, column tile | k-step << 8) of its degree.
+__global__ void __launch_bounds__(64)
+pack_go_gen_kernel(const float2* __restrict__ gO, const int* __restrict__ map, float* __restrict__ Bg, int nO, int nBg) {
+    const int* mp = map + 4 * blockIdx.x;
+    const int cumO = mp[0], M = mp[1], tO = mp[2], ks = mp[3] >> 8;
+    const int ct = mp[3] & 255;
+    const int lane = threadIdx.x, i = lane & 15, kk = lane >> 4;
+    const int k = 4 * ks + kk, to = k >> 1, sel = k & 1;
+    const int col = 16 * ct + i, m = col >> 1, r = col & 1;
+    float v = 0.f;
+    if (to < tO && m < M) {
+        const float2 z = gO[(size_t)blockIdx.y * nO + cumO + to * M + m];
+        v = (r == sel) ? (r ? -z.x : z.x) : z.y;
+    }
+    Bg[(size_t)blockIdx.y * nBg + (size_t)blockIdx.x * 64 + lane] = v;
 }
 
 // Builds the operands the unit kernel copies straight into LDS: fragments with one zero behind
@@ -1274,6 +1635,10 @@ static void free_plan(cgnet_cg_plan* plan) {
     if (plan->d_bwd_utasks) (void)hipFree(plan->d_bwd_utasks);
     if (plan->d_bwd_combine) (void)hipFree(plan->d_bwd_combine);
     if (plan->d_bwd_padmeta) (void)hipFree(plan->d_bwd_padmeta);
+    if (plan->d_gens) (void)hipFree(plan->d_gens);
+    if (plan->d_ftasks) (void)hipFree(plan->d_ftasks);
+    if (plan->d_packmap) (void)hipFree(plan->d_packmap);
+    if (plan->d_bmap) (void)hipFree(plan->d_bmap);
     delete plan;
 }
 
@@ -1967,5 +2332,188 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
                            (const float2*)d_workspace, (float2*)d_gF, n, ng);
         CGNET_HIP(hipGetLastError());
     }
+    return CGNET_OK;
+}
+
+// ---- fused layer backward: host side -----------------------------------------------------------
+// Links the product plan with a mixing plan: per-task metadata on the device, rebuilt only when the mixing
+// plan's per-degree layout differs from the one linked last.  Returns CGNET_ERR_UNSUPPORTED (with the reason) for
+// shapes the fused kernel does not take.
+static int link_fused(const cgnet_cg_plan* p, const cgnet_wmm_plan* w) {
+    CGNET_REQUIRE(p->bwd_fast && p->bwd_hybrid, CGNET_ERR_UNSUPPORTED,
+                  "the fused backward needs the matrix-core unit backward (every channel count in 8..16, lmax <= 23)");
+    CGNET_REQUIRE(wmm_gradff_operand_ok(w), CGNET_ERR_UNSUPPORTED, "the fused backward needs t_O <= 16 in every degree");
+    CGNET_REQUIRE(wmm_plan_degrees(w) == p->L + 1, CGNET_ERR_ARG, "the two plans have different lmax");
+    std::vector<int> sig;
+    std::vector<WmmDegInfo> info(p->L + 1);
+    for (int l = 0; l <= p->L; ++l) {
+        if (int rc = wmm_plan_degree(w, l, &info[l])) return rc;
+        CGNET_REQUIRE(info[l].K == p->t_FF[l], CGNET_ERR_ARG,
+                      "degree %d: the mixing plan has %d mid channels, the product %d", l, info[l].K, p->t_FF[l]);
+        const int v[4] = {info[l].tO, info[l].cumO, info[l].cumW, info[l].cumT};
+        sig.insert(sig.end(), v, v + 4);
+    }
+    std::lock_guard<std::mutex> lock(p->fused_mu);
+    if (p->d_gens && sig == p->fused_signature) return CGNET_OK;
+    // packed B operand of one sample: per degree nct x nks blocks of 64 floats
+    std::vector<int> boff(p->L + 1, 0), bmap;
+    int bop = 0, bcap = 16;
+    for (int l = 0; l <= p->L; ++l) {
+        const int M = 2 * l + 1, nct = (2 * M + 15) / 16, nks = info[l].tO > 0 ? (2 * info[l].tO + 3) / 4 : 0;
+        boff[l] = bop;
+        if (p->t_FF[l] == 0) continue;
+        for (int ct = 0; ct < nct; ++ct)
+            for (int ks = 0; ks < nks; ++ks) {
+                const int v[4] = {info[l].cumO, M, info[l].tO, ct | (ks << 8)};
+                bmap.insert(bmap.end(), v, v + 4);
+            }
+        bop += nct * nks * 64;
+        bcap = std::max(bcap, nct * nks * 256);
+    }
+    std::vector<GenTask> gens(p->bwd_utasks.size());
+    std::vector<FusedTask> ft(p->bwd_utasks.size());
+    std::vector<int> map;
+    size_t aoff = 0;
+    int acap = 16;
+    for (const BwdUnit& u : p->bwd_units) {
+        for (int k = u.task_begin; k < u.task_end; ++k) {
+            const BwdUTask& t = p->bwd_utasks[k];
+            const WmmDegInfo& d = info[t.l];
+            const int M = 2 * t.l + 1, nct = (2 * M + 15) / 16;
+            GenTask g{};
+            g.aoff = (int)aoff;
+            g.nks = d.tO > 0 ? (2 * d.tO + 3) / 4 : 0;
+            g.tO = d.tO;
+            g.chan0 = (t.offFF - p->cumFF[t.l]) / M;
+            g.nch = u.rows * t.tau2;
+            g.cumW = d.cumW;
+            g.K = d.K;
+            g.cumT = d.cumT;
+            gens[k] = g;
+            const int nrt = (g.nch + 15) / 16;
+            for (int rt = 0; rt < nrt && g.nks > 0; ++rt) { map.push_back(k); map.push_back(rt); }
+            FusedTask f{};
+            f.geom = t.l | (t.l2 << 8) | (t.tau2 << 16) | (t.first_of_l2 << 24) | (t.last_of_l2 << 25);
+            f.offF2p = t.offF2p;
+            f.cgp_off = t.cgp_off;
+            f.cgp_len = t.cgp_len;
+            f.p2off = t.p2off;
+            f.aoff = g.aoff;
+            f.shape = g.nks | (d.tO << 8) | (g.nch << 16);
+            f.boff = boff[t.l];
+            const int nkp = (g.nks + 1) / 2;
+            f.chunks = (nrt * 32 * nkp) | ((nct * g.nks * 16) << 16);     // 16-byte pieces of the A block | of the B block
+            ft[k] = f;
+            aoff += (size_t)nrt * 128 * nkp;
+            CGNET_REQUIRE(aoff < (1u << 30), CGNET_ERR_UNSUPPORTED, "packed weights of the fused backward exceed 2^30 floats");
+            acap = std::max(acap, nrt * 512 * nkp);
+        }
+    }
+    const size_t lds = bwd_fused_lds(p->bwd_f1cap, p->bwd_f2cap, p->bwd_cgcap, p->bwd_tcap, bcap, acap);
+    CGNET_REQUIRE(lds <= kMaxHybLds, CGNET_ERR_UNSUPPORTED,
+                  "the fused backward would need %zu bytes of LDS per work-group (limit %zu)", lds, kMaxHybLds);
+    // synchronous copies: kernels of an earlier call that still read the old entries have finished when they return
+    CGNET_HIP(hipDeviceSynchronize());
+    auto upload = [](const void* src, size_t bytes, void** dst) -> int {
+        if (*dst) { (void)hipFree(*dst); *dst = nullptr; }
+        if (bytes == 0) return CGNET_OK;
+        CGNET_HIP(hipMalloc(dst, bytes));
+        CGNET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return CGNET_OK;
+    };
+    if (int rc = upload(gens.data(), sizeof(GenTask) * gens.size(), (void**)&p->d_gens)) return rc;
+    if (int rc = upload(ft.data(), sizeof(FusedTask) * ft.size(), (void**)&p->d_ftasks)) return rc;
+    if (int rc = upload(map.data(), sizeof(int) * map.size(), (void**)&p->d_packmap)) return rc;
+    if (int rc = upload(bmap.data(), sizeof(int) * bmap.size(), (void**)&p->d_bmap)) return rc;
+    p->fused_npack = (int)(map.size() / 2);
+    p->fused_nbmap = (int)(bmap.size() / 4);
+    p->fused_operand_floats = aoff;
+    p->fused_bop_floats = bop;
+    p->fused_signature = sig;
+    p->fused_bcap = bcap;
+    p->fused_acap = acap;
+    if (int rc = raise_dynamic_lds((const void*)cgbn_backward_fused_kernel, lds)) return rc;
+    return CGNET_OK;
+}
+
+extern "C" int cgnet_CGBN_backward_fused_supported(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan) {
+    clear_error();
+    if (!cg_plan || !wmm_plan) return 0;
+    return link_fused(cg_plan, wmm_plan) == CGNET_OK ? 1 : 0;
+}
+
+static size_t fused_workspace_parts(const cgnet_cg_plan* p, int B, size_t* a_off, size_t* b_off) {
+    size_t o = cgnet_sparse_backward_workspace(p, B);
+    *a_off = o;
+    o += align_up(sizeof(float) * p->fused_operand_floats, 256);
+    *b_off = o;
+    o += align_up(sizeof(float) * (size_t)p->fused_bop_floats * B, 256);
+    return o;
+}
+
+extern "C" size_t cgnet_CGBN_backward_fused_workspace(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, int B) {
+    if (!cg_plan || !wmm_plan || B <= 0 || !cg_plan->bwd_fast) return 0;
+    if (link_fused(cg_plan, wmm_plan) != CGNET_OK) return 0;
+    size_t a, b;
+    return fused_workspace_parts(cg_plan, B, &a, &b);
+}
+
+extern "C" int cgnet_CGBN_backward_fused(const cgnet_cg_plan* plan, const cgnet_wmm_plan* wmm_plan, const float* d_F,
+                                         float* d_gF, const float* d_gO, const float* d_W, const float* d_CG, int B,
+                                         const float* d_stds, float eps, int flags, void* d_workspace,
+                                         size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan && wmm_plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    if (B == 0 || plan->nF == 0) return CGNET_OK;
+    if (int rc = link_fused(plan, wmm_plan)) return rc;
+    const bool bn = flags & CGNET_FN_BATCHNORM;
+    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    CGNET_REQUIRE(d_F && d_gF && d_gO && d_W && d_CG, CGNET_ERR_ARG, "null device pointer");
+    CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
+    size_t a_off, b_off;
+    const size_t need = fused_workspace_parts(plan, B, &a_off, &b_off);
+    CGNET_REQUIRE(d_workspace && workspace_bytes >= need, CGNET_ERR_WORKSPACE,
+                  "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    CGNET_REQUIRE(((uintptr_t)d_workspace & 15) == 0, CGNET_ERR_ARG, "workspace must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    float2* part1 = (float2*)d_workspace;
+    float2* part2 = (float2*)((char*)part1 + align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256));
+    float2* Fp = (float2*)((char*)part2 + align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256));
+    float* CGP = (float*)((char*)Fp + align_up(sizeof(float) * 2 * (size_t)plan->bwd_nFp * B, 256));
+    float* Ag = (float*)((char*)d_workspace + a_off);
+    float* Bg = (float*)((char*)d_workspace + b_off);
+    WmmDegInfo last;
+    if (int rc = wmm_plan_degree(wmm_plan, plan->L, &last)) return rc;
+    const int nO = last.cumO + last.tO * (2 * plan->L + 1);
+    if (plan->fused_npack > 0) {
+        CGNET_LAUNCH(pack_w_gen_kernel, dim3((unsigned)plan->fused_npack), dim3(64), 0, s, (const float2*)d_W,
+                     bn ? d_stds : nullptr, eps, plan->d_gens, plan->d_packmap, Ag);
+        CGNET_HIP(hipGetLastError());
+    }
+    if (plan->fused_nbmap > 0) {
+        CGNET_LAUNCH(pack_go_gen_kernel, dim3((unsigned)plan->fused_nbmap, (unsigned)B), dim3(64), 0, s,
+                     (const float2*)d_gO, plan->d_bmap, Bg, nO, plan->fused_bop_floats);
+        CGNET_HIP(hipGetLastError());
+    }
+    const size_t npad = (size_t)plan->bwd_nFp * B;
+    const int nbF = (int)((npad + 255) / 256);
+    CGNET_LAUNCH(cg_backward_pad_kernel, dim3((unsigned)(nbF + plan->nllls)), dim3(256), 0, s,
+                 (const float2*)d_F, d_CG, Fp, CGP, plan->d_bwd_padmeta, plan->L, plan->nF, plan->bwd_nFp, B, nbF);
+    CGNET_HIP(hipGetLastError());
+    CGNET_REQUIRE((long long)B * (long long)plan->bwd_units.size() < (1LL << 31), CGNET_ERR_UNSUPPORTED,
+                  "%d samples x %zu units exceed the grid limit", B, plan->bwd_units.size());
+    const size_t lds = bwd_fused_lds(plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, plan->fused_bcap,
+                                     plan->fused_acap);
+    CGNET_LAUNCH(cgbn_backward_fused_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads), lds, s,
+                 (const float2*)Fp, (const float*)Bg, (const float*)Ag, (const float*)CGP, part1, part2,
+                 plan->d_bwd_units, plan->d_ftasks, plan->nF, plan->bwd_nFp, plan->fused_bop_floats, plan->bwd_P2,
+                 plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, plan->fused_bcap, plan->fused_acap, B);
+    CGNET_HIP(hipGetLastError());
+    const size_t n = (size_t)plan->nF * B;
+    CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+                 (const float2*)part1, (const float2*)part2, (float2*)d_gF, plan->d_bwd_combine, plan->L,
+                 plan->nF, plan->bwd_P2, B);
+    CGNET_HIP(hipGetLastError());
     return CGNET_OK;
 }

@@ -41,6 +41,12 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Returns CGNET_OK or CGNET_ERR_HIP (message recorded).
 int raise_dynamic_lds(const void* func, size_t bytes);
 
+// ---- what the fused layer backward (CG product side) needs to know of a mixing plan -----------
+struct WmmDegInfo { int K, tO, cumO, cumW, cumT; };                 // per degree: mid / output channels, offsets of gO, W, stds
+bool wmm_gradff_operand_ok(const cgnet_wmm_plan* plan);             // every degree has t_O <= 16
+int wmm_plan_degrees(const cgnet_wmm_plan* plan);                   // L + 1
+int wmm_plan_degree(const cgnet_wmm_plan* plan, int l, WmmDegInfo* info);
+
 // Optional per-kernel timing (cgnet_profile_*): when enabled, every launch is bracketed by a
 // pair of HIP events recorded on the launch stream.
 class KernelTimer {

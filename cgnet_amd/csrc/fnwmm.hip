@@ -1072,6 +1072,17 @@ extern "C" int cgnet_FN_WMM_forward(const cgnet_wmm_plan* plan, const float* d_F
     return CGNET_OK;
 }
 
+namespace cgnet {
+bool wmm_gradff_operand_ok(const cgnet_wmm_plan* plan) { return plan && plan->gff_mfma; }
+int wmm_plan_degrees(const cgnet_wmm_plan* plan) { return (int)plan->degs.size(); }
+int wmm_plan_degree(const cgnet_wmm_plan* plan, int l, WmmDegInfo* info) {
+    if (!plan || l < 0 || l >= (int)plan->degs.size() || !info) return CGNET_ERR_ARG;
+    const WmmDeg& d = plan->degs[l];
+    *info = WmmDegInfo{d.K, d.tO, d.cumO, d.cumW, d.cumT};
+    return CGNET_OK;
+}
+}  // namespace cgnet
+
 static int gradw_chunks(int B) { return (B + kGradWChunk - 1) / kGradWChunk; }
 static size_t gff_operand_bytes(const cgnet_wmm_plan* plan) {
     return plan->gff_mfma ? sizeof(float) * 64 * (size_t)plan->ap_blocks : sizeof(float) * 2 * (size_t)plan->nW;

@@ -157,6 +157,26 @@ int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* 
                           float eps, int flags,
                           void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* ---- the whole layer's backward in one pass (no counterpart in the reference) -------------------- */
+
+/* gF = dLoss/dF of  F -> CG product -> fragment norm + weight mixing -> O  from d_gO = dLoss/dO, i.e. what
+ * cgnet_FN_WMM_backward(d_gFF = ...) followed by cgnet_sparse_backward(d_gFF) returns in d_gF, bit for bit,
+ * without the intermediate gradient gFF (B x nFF complex) ever existing in memory: every tile of it is formed
+ * in LDS on the matrix cores from gO and conj(W)/div right where the product's backward consumes it.  The
+ * reference has no such call (its two autograd Functions meet at a materialised grad_FF,
+ * CGNet/CG_layers.py:54-72,194-203); it is legal wherever FF is not visible to the user, i.e. inside
+ * CGBN_cuda.forward (CG_layers.py:313-318).  The weight gradient still comes from cgnet_FN_WMM_backward
+ * (d_gFF = NULL).  cgnet_CGBN_backward_fused_supported returns 1 for the shapes the fused kernel takes
+ * (every input channel count in 8..16, lmax <= 23, t_O <= 16, LDS within limits) and 0 otherwise, with
+ * cgnet_last_error() naming the reason; the call itself then returns CGNET_ERR_UNSUPPORTED.
+ * d_stds / eps / flags as in cgnet_FN_WMM_backward (the stds the forward pass used, treated as constants). */
+int cgnet_CGBN_backward_fused_supported(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan);
+size_t cgnet_CGBN_backward_fused_workspace(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, int B);
+int cgnet_CGBN_backward_fused(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, const float* d_F,
+                              float* d_gF, const float* d_gO, const float* d_W, const float* d_CG, int B,
+                              const float* d_stds, float eps, int flags,
+                              void* d_workspace, size_t workspace_bytes, void* stream);
+
 /* ---- measurement hooks (no counterpart in the reference, which times nothing) ------------ */
 
 /* With timing enabled every kernel launch of this library is bracketed by two HIP events

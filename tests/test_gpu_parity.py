@@ -438,11 +438,15 @@ def check_layer_step(dev, mod, ora, twin, w64, x64, go64):
     return x
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["fused_backward", True, False])
 @pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn", LAYER_CASES)
 def test_layer_forward_backward(dev, lmax, tin, tout, bsz, sparse, bn, fused):
+    """fused: one autograd node for the layer (statistics inside the product kernel); "fused_backward": in addition the
+    backward runs from grad_output to the input gradient in one kernel where the shapes allow it (the two 11-degree
+    cases here), without grad_FF in memory; False: the reference's two Functions chained."""
     mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=lmax + bsz)
-    mod.fused = fused
+    mod.fused = bool(fused)
+    mod.fused_backward = fused == "fused_backward"
     x64 = rand_straight(tin, bsz, seed=21)
     g = torch.Generator().manual_seed(23)
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
@@ -481,6 +485,56 @@ def test_layer_config5_shape(dev):
     x64 = rand_straight(tau, 1, seed=22)
     go64 = randn32((1, 16 * 441, 2), torch.Generator().manual_seed(24))
     check_layer_step(dev, mod, ora, twin, w64, x64, go64)
+
+
+def _fused_backward_cases(n, seed):
+    """Layers whose backward the one-kernel route takes: every input channel count in 8..16, at most 16 outputs."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for k in range(n):
+        lmax = int(rng.integers(0, 8))
+        tin = [int(rng.integers(8, 17)) for _ in range(lmax + 1)]
+        tout = [int(rng.integers(0, 17)) for _ in range(lmax + 1)]
+        cases.append((lmax, tin, tout, int(rng.integers(1, 7)), bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0), k))
+    return cases + [(11, [12] * 12, [12] * 12, 2, False, True, n), (15, [16] * 16, [16] * 16, 1, True, True, n + 1),
+                    (20, [16] * 21, [16] * 21, 1, False, True, n + 2)]
+
+
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _fused_backward_cases(12, 31))
+def test_fused_backward_equals_two_kernel_backward(dev, lmax, tin, tout, bsz, sparse, bn, k):
+    """The one-kernel backward (gFF tiles formed in LDS) returns bit for bit what the gFF kernel followed by the
+    product's backward returns, for the input gradient and the weight gradient, in training mode; the small
+    cases are also held against the oracle."""
+    from cgnet_amd import _plans
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=400 + k)
+    if not _plans.fused_backward_supported(mod.cg.native_plan(), mod.bnWMM.native_plan()):
+        from cgnet_amd import _lib
+        pytest.skip("shape not taken by the fused backward: " + _lib.load().cgnet_last_error().decode())
+    x64 = rand_straight(tin, bsz, seed=500 + k)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go = randn32((bsz, n_o, 2), torch.Generator().manual_seed(600 + k)).float().to(dev)
+    stds0 = mod.bnWMM.bn_stds.detach().clone() if bn else None
+    grads = []
+    for fb in (False, True):
+        mod.fused_backward = fb
+        mod.bnWMM.bn_cnt = 1.0
+        if bn:
+            with torch.no_grad():
+                mod.bnWMM.bn_stds.copy_(stds0)
+        mod.bnWMM.W.grad = None
+        x = x64.float().to(dev).requires_grad_(True)
+        mod(x, straight_output=True).backward(go)
+        grads.append((x.grad.clone(), mod.bnWMM.W.grad.clone() if mod.bnWMM.W.numel() else None))
+    assert torch.equal(grads[0][0], grads[1][0]), "input gradient differs: max %.3e" % float((grads[0][0] - grads[1][0]).abs().max())
+    if grads[0][1] is not None:
+        assert torch.equal(grads[0][1], grads[1][1])
+    if lmax <= 8:
+        if bn:
+            with torch.no_grad():
+                mod.bnWMM.bn_stds.copy_(stds0)
+        mod.bnWMM.bn_cnt = 1.0
+        mod.fused_backward = True
+        check_layer_step(dev, mod, ora, twin, w64, x64, go.double().cpu())
 
 
 def _random_layer_cases(n, seed, out_lo=1):
