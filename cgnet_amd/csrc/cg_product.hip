@@ -49,6 +49,7 @@ struct BwdUnit {
     int task_begin, task_end; // range in the unit-ordered task array (sorted by l2, then l)
     int nA;                   // waves that take slot 1; the other waves of the group take slot 2
     int TI, RW;               // slot-1 tiling: output rows per thread, lanes sharing one output
+    int RM;                   // of those RW lanes, RM (1 or 2) split the reduced m range, RW / RM the reduced channels
     int p1off;                // slot-1 result: -1 = the unit's rows in the slot-1 area, else offset of its rows in the
                               // slot-2 partial area (a degree whose task list is split over several units)
 };
@@ -101,6 +102,7 @@ struct cgnet_cg_plan {
     std::vector<int> bwd_group_table_off;        // for ng groups: first entry of its ng+1 boundaries
     int* d_bwd_group_table = nullptr;
     size_t fwd_lds = 0, bwd_lds = 0;
+    bool fwd_mm = false;                         // the forward runs cg_forward_mm_kernel (product on the matrix cores)
     std::vector<int> fwd_class_begin;            // forward tasks by LDS class: class k = tasks [begin[k], begin[k+1])
     std::vector<size_t> fwd_class_lds;           // LDS bytes of a work-group of class k
     int bwd_threads = 256;                       // work-group size of the backward kernel
@@ -397,6 +399,173 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
 #undef CGNET_FWD
 }
 
+// ---- forward on the matrix cores ---------------------------------------------------------------
+// For a fixed output m the tile's channels are a small matrix product:
+//   FF_m[t1, t2] = sum_m2 (C[m][m2] F1[t1][m - m2]) * F2[t2][m2]              (rows x terms) . (terms x tau2)
+// rows of the accumulator = the up to 16 rows of the task, columns = the up to 16 channels of degree l2, the
+// reduction runs over the valid m2 in steps of four (v_mfma_f32_16x16x4_f32; complex numbers as four real
+// products per step).  Only the left operand needs arithmetic (one coefficient times one fragment entry per lane
+// and step); the right operand is read as it lies in the staged l2 slab.  No masking: the table is staged with three
+// zeros behind every row, and holds zeros where m - m2 is no valid m1 (every table this library fills does), so the
+// steps past the last valid m2 multiply whatever finite fragment entries lie next to the rows by zero (LDS is
+// cleared once, the slabs have 32 spare bytes on either side).  Every wave takes every fourth m, numbered from
+// the middle outwards, and writes its 16 x 16 results into the output tile; the tile then leaves as in the
+// vector-ALU kernel.  Used when every channel count is in 8..16.
+constexpr int kFwdMmPad = 32;     // bytes before / between / behind the fragment buffers
+
+__host__ __device__ inline size_t fwd_task_lds_mm(const CgTask& t) {
+    const size_t M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
+    return kFwdMmPad + 2 * (fwd_frag_lds(t) + kFwdMmPad) + ((8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15) +
+           ((4 * M * (M2 + 3) + 15) & ~(size_t)15);
+}
+
+// One sample of a task: the waves take the values of m in turn (from the middle outwards, so that every wave gets
+// long and short ones); for one m the accumulator D[t1][t2] gathers the steps of four m2.
+__device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __restrict__ cg, int P,
+                                              const float2* __restrict__ f1, const float2* __restrict__ f2,
+                                              float2* __restrict__ out, int wave, int nwaves, int lane) {
+    const int l = t.l, l1 = t.l1, l2 = t.l2;
+    const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
+    const int rows = t.rows, tau2 = t.tau2;
+    const int i = lane & 15, kk = lane >> 4;
+    // rows / channels past the end repeat the last one (their results are not stored)
+    const unsigned a_row = lds_addr(f1 + min(i, rows - 1) * M1);
+    const unsigned b_row = lds_addr(f2 + min(i, tau2 - 1) * M2);
+    const unsigned c_lane = lds_addr(cg + kk);
+    for (int mslot = wave; mslot < M; mslot += nwaves) {
+        const int mm = (mslot & 1) ? l + ((mslot + 1) >> 1) : l - (mslot >> 1);
+        const int m = mm - l;
+        const int lo = max(-l2, m - l1), hi = min(l2, m + l1);
+        const int nsteps = (hi - lo + 4) >> 2;
+        // lane kk of a step takes m2 = lo + 4 s + kk, i.e. m1 = m - m2; past hi the table pitch holds zeros and the
+        // fragment reads stay inside the padded buffers
+        unsigned pa = opaque(a_row + 8u * (unsigned)(m - lo + l1 - kk));
+        unsigned pb = opaque(b_row + 8u * (unsigned)(lo + l2 + kk));
+        unsigned pc = opaque(c_lane + 4u * (unsigned)(mm * P + lo + l2));
+        f32x4 dre = {0.f, 0.f, 0.f, 0.f}, dim = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < nsteps; ++s) {
+            const float c = lds_f(pc)[0];
+            const float2 fa = lds_c(pa, 0), fb = lds_c(pb, 0);
+            pa -= 32u;
+            pb += 32u;
+            pc += 16u;
+            const float ar = c * fa.x, ai = c * fa.y, nai = -ai;
+            dre = mfma4(ar, fb.x, dre);
+            dim = mfma4(ar, fb.y, dim);
+            dre = mfma4(nai, fb.y, dre);
+            dim = mfma4(ai, fb.x, dim);
+        }
+        mfma_drain();
+        if (i < tau2) {
+            float2* o = out + (4 * kk * tau2 + i) * M + mm;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (4 * kk + v < rows) o[v * tau2 * M] = make_float2(dre[v], dim[v]);
+        }
+    }
+}
+
+constexpr int kFwdMmThreads = 512;
+
+__global__ void __launch_bounds__(kFwdMmThreads)
+cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const float* __restrict__ CG,
+                     const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
+                     double* __restrict__ stats_part, int sumT, int lds_bytes) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const UnitPart up = part_major((B + samples_per_group - 1) / samples_per_group);
+    const CgTask t = tasks[up.unit];
+    const int group = up.part;
+    const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
+    const int P = M2 + 3;
+    const int nch = t.rows * t.tau2;
+    const int nout = nch * M, n1 = t.rows * M1, n2 = t.tau2 * M2;
+    const size_t out_bytes = (8 * (size_t)nout + 15) & ~(size_t)15;
+    const size_t f1_bytes = (8 * (size_t)n1 + 15) & ~(size_t)15;
+    const size_t frag_bytes = fwd_frag_lds(t) + kFwdMmPad;          // one buffer and the pad behind it
+    unsigned char* frag = smem + kFwdMmPad;                        // [2][frag_bytes]
+    float2* out = reinterpret_cast<float2*>(frag + 2 * frag_bytes);
+    float* cg = reinterpret_cast<float*>(frag + 2 * frag_bytes + out_bytes);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    {
+        float4* z = reinterpret_cast<float4*>(smem);
+        for (int e = tid; e < (lds_bytes >> 4); e += kFwdMmThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __syncthreads();                                               // the clearing stores precede every copy
+    auto issue = [&](int b, int par) {
+        const float2* Fb = F + (size_t)b * nF;
+        unsigned char* d1 = frag + par * frag_bytes;
+        unsigned char* d2 = d1 + f1_bytes;
+        dma16<kFwdMmThreads>(Fb + t.offF1, d1, n1 >> 1, tid);
+        if (n1 & 1) dma8(Fb + t.offF1 + (n1 - 1), d1 + 8 * (size_t)(n1 - 1), tid);
+        dma16<kFwdMmThreads>(Fb + t.offF2, d2, n2 >> 1, tid);
+        if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
+    };
+    double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};
+    const int b0 = group * samples_per_group;
+    const int b1 = min(B, b0 + samples_per_group);
+    if (b0 < b1) issue(b0, 0);
+    // the table with three zeros behind every row (the zeros are the cleared LDS)
+    for (int e = tid; e < M * M2; e += kFwdMmThreads) {
+        const int r = e / M2;
+        cg[r * P + (e - r * M2)] = CG[t.cg_off + e];
+    }
+    int par = 0;
+    for (int b = b0; b < b1; ++b, par ^= 1) {
+        dma_wait();
+        __syncthreads();       // this sample's fragments landed; the previous tile has been copied out
+        if (b + 1 < b1) issue(b + 1, par ^ 1);
+        const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
+        const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
+#ifndef CGNET_TEST_FWD_NOCOMPUTE
+        fwd_mm_sample(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane);
+#endif
+        __syncthreads();
+        // tile -> FF with 16-byte stores from the first 16-byte boundary on
+        float2* dst = FF + (size_t)b * nFF + t.offFF;
+        const int head = min(nout, (int)((reinterpret_cast<uintptr_t>(dst) >> 3) & 1));
+        const int npair = (nout - head) >> 1;
+        float4* dst4 = reinterpret_cast<float4*>(dst + head);
+#ifndef CGNET_TEST_FWD_NOSTORE
+        for (int e = tid; e < npair; e += kFwdMmThreads) {
+            const float2 u = out[head + 2 * e], v = out[head + 2 * e + 1];
+            stream_store16(dst4 + e, u.x, u.y, v.x, v.y);
+        }
+#endif
+        if (tid == 0 && head) dst[0] = out[0];
+        if (tid == 1 && ((nout - head) & 1)) dst[nout - 1] = out[nout - 1];
+        if (stats_part) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int ch = tid + kFwdMmThreads * k;
+                if (ch < nch) {
+                    // both sums run over the same rounded |z| in double (see cg_forward_kernel)
+                    double a = s1[k], q = s2[k];
+                    for (int mm = 0; mm < M; ++mm) {
+                        const float2 z = out[ch * M + mm];
+                        const double r = (double)sqrt_hw(fmaf(z.x, z.x, z.y * z.y));
+                        a += r;
+                        q = fma(r, r, q);
+                    }
+                    s1[k] = a;
+                    s2[k] = q;
+                }
+            }
+        }
+    }
+    if (stats_part) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int ch = tid + kFwdMmThreads * k;
+            if (ch < nch) {
+                double* p = stats_part + ((size_t)group * sumT + t.chan0 + ch) * 2;
+                p[0] = s1[k];
+                p[1] = s2[k];
+            }
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256)
 stats_reduce_kernel(const double* __restrict__ part, double* __restrict__ sums, int n2, int ngroups) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -660,7 +829,7 @@ constexpr int kTabLo = 1, kTabHi = 2;
 // layout as bwd_phase, one item per thread (rtid = thread index inside its role), no reduction.
 // g: the tile exactly as it lies in gFF ([t1][t2][m], no padding); cgp: the table with kTabLo /
 // kTabHi zero rows; fr: fragment rows of the reduced slot with one trailing zero each.
-template <int SLOT, int TI, int RW>
+template <int SLOT, int TI, int RW, int RM = 1>
 __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restrict__ cgp,
                                           const float2* __restrict__ g, const float2* __restrict__ fr,
                                           int rtid, float (&ax)[kBwdMaxTI][2], float (&ay)[kBwdMaxTI][2]) {
@@ -673,15 +842,24 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     const int g_so = (SLOT == 1) ? tau2 * M : M;
     const int g_sr = (SLOT == 1) ? M : tau2 * M;
     const int d = l1 + l2 - l;
-    const int item = rtid / RW, lane_r = rtid % RW;
+    // the RW lanes of an item: RM of them split the reduced m range (the first takes an even number of steps, so
+    // that its two-step loop ends exactly where the second begins), RW / RM split the reduced channels
+    constexpr int RC = RW / RM;
+    static_assert(RM == 1 || (RM == 2 && RW % 2 == 0), "the reduced m range is split in two at most");
+    const int item = rtid / RW, lane_r = (rtid % RW) % RC, lane_m = (rtid % RW) / RC;
     const int nT = (n_o + TI - 1) / TI;
     const int nWin = (M_o + 1) >> 1;
     if (item >= nT * nWin) return;
     int w, to;
     bwd_item(item, nT, nWin, w, to);
     const int mo0 = 2 * w;
-    const int ir_lo = max(0, d - mo0 - 1);
-    const int ir_hi = min(M_r - 1, M - 1 + d - mo0);
+    int ir_lo = max(0, d - mo0 - 1);
+    int ir_hi = min(M_r - 1, M - 1 + d - mo0);
+    if (RM == 2) {
+        const int first = (((ir_hi - ir_lo + 1) >> 1) + 1) & ~1;      // about half, even
+        if (lane_m == 0) ir_hi = min(ir_hi, ir_lo + first - 1);
+        else ir_lo = ir_lo + first;
+    }
     int go[TI];
 #pragma unroll
     for (int i = 0; i < TI; ++i) go[i] = min(to + nT * i, n_o - 1) * g_so;
@@ -690,7 +868,7 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     // step pair (ir, ir+1):  c0 = T[p][k0], c1 = T[p+1][k1], c0' = T[p+1][k0'], c1' = T[p+2][k1']
     // with p the table row of (mo0, ir); slot 1: k = ir (k0' = k1' = ir+1), slot 2: k0 = col0, k1 = col1.
     const unsigned c_step = (SLOT == 1) ? 8u * (M2 + 1) : 8u * M2;     // two rows (and two columns) per pair
-    for (int r = lane_r; r < n_r; r += RW) {
+    for (int r = lane_r; r < n_r; r += RC) {
         unsigned gp[TI];
 #pragma unroll
         for (int i = 0; i < TI; ++i) gp[i] = lds_addr(g + r * g_sr + (mo0 - d) + go[i] + ir_lo);
@@ -818,6 +996,45 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         default: { CALL(4, 16); } break;                                         \
     }
 
+// slot-1 tilings: as above, plus the variants whose lanes also split the reduced m range in two
+#define CGNET_BWD_SWITCH_A(TI_, RW_, RM_, CALL)                                  \
+    if ((RM_) == 2) {                                                            \
+        switch ((TI_) * 32 + (RW_)) {                                            \
+            case 2 * 32 + 4: { CALL(2, 4, 2); } break;                           \
+            case 2 * 32 + 8: { CALL(2, 8, 2); } break;                           \
+            case 2 * 32 + 16: { CALL(2, 16, 2); } break;                         \
+            case 3 * 32 + 4: { CALL(3, 4, 2); } break;                           \
+            case 3 * 32 + 8: { CALL(3, 8, 2); } break;                           \
+            case 3 * 32 + 16: { CALL(3, 16, 2); } break;                         \
+            case 4 * 32 + 4: { CALL(4, 4, 2); } break;                           \
+            case 4 * 32 + 8: { CALL(4, 8, 2); } break;                           \
+            default: { CALL(4, 16, 2); } break;                                  \
+        }                                                                        \
+    } else {                                                                     \
+        switch ((TI_) * 32 + (RW_)) {                                            \
+            case 1 * 32 + 1: { CALL(1, 1, 1); } break;                           \
+            case 1 * 32 + 2: { CALL(1, 2, 1); } break;                           \
+            case 1 * 32 + 4: { CALL(1, 4, 1); } break;                           \
+            case 1 * 32 + 8: { CALL(1, 8, 1); } break;                           \
+            case 1 * 32 + 16: { CALL(1, 16, 1); } break;                         \
+            case 2 * 32 + 1: { CALL(2, 1, 1); } break;                           \
+            case 2 * 32 + 2: { CALL(2, 2, 1); } break;                           \
+            case 2 * 32 + 4: { CALL(2, 4, 1); } break;                           \
+            case 2 * 32 + 8: { CALL(2, 8, 1); } break;                           \
+            case 2 * 32 + 16: { CALL(2, 16, 1); } break;                         \
+            case 3 * 32 + 1: { CALL(3, 1, 1); } break;                           \
+            case 3 * 32 + 2: { CALL(3, 2, 1); } break;                           \
+            case 3 * 32 + 4: { CALL(3, 4, 1); } break;                           \
+            case 3 * 32 + 8: { CALL(3, 8, 1); } break;                           \
+            case 3 * 32 + 16: { CALL(3, 16, 1); } break;                         \
+            case 4 * 32 + 1: { CALL(4, 1, 1); } break;                           \
+            case 4 * 32 + 2: { CALL(4, 2, 1); } break;                           \
+            case 4 * 32 + 4: { CALL(4, 4, 1); } break;                           \
+            case 4 * 32 + 8: { CALL(4, 8, 1); } break;                           \
+            default: { CALL(4, 16, 1); } break;                                  \
+        }                                                                        \
+    }
+
 struct BwdCtx {
     const float2* Fp;          // this sample's fragments, rows padded with one zero
     const float2* Gb;          // this sample's gFF
@@ -866,7 +1083,7 @@ __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int
 }
 
 // Waves of role A: gradient of slot 1 (rows of degree l1), kept in registers for the whole unit.
-template <int NT, int TI, int RW>
+template <int NT, int TI, int RW, int RM>
 __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdUTask t,
                                                 float2* __restrict__ dst) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
@@ -883,7 +1100,7 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         bwd_stage<NT>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
 #ifndef CGNET_TEST_NOSLOT1
-        bwd_accum<1, TI, RW>(q, cgp, g, f2, c.rtid, ax, ay);
+        bwd_accum<1, TI, RW, RM>(q, cgp, g, f2, c.rtid, ax, ay);
 #endif
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
@@ -970,8 +1187,8 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
     // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
-#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<kThreads, TI_, RW_>(c, u, t0, dst)
-        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kThreads, TI_, RW_, RM_>(c, u, t0, dst)
+        CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
         bwd_unit_loop_b(c, u, t0, part2 + (size_t)b * P2);
@@ -1172,8 +1389,8 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
     // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
-#define CGNET_LOOP_A(TI_, RW_) bwd_unit_loop_a<kHybThreads, TI_, RW_>(c, u, t0, dst)
-        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kHybThreads, TI_, RW_, RM_>(c, u, t0, dst)
+        CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
         bwd_hybrid_loop_b(c, u, t0, wave - u.nA, kHybWaves - u.nA, tid & 63, part2 + (size_t)b * P2);
@@ -1337,7 +1554,7 @@ __device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTa
 }
 
 // Waves of role A (slot 1 on the vector ALUs), as bwd_unit_loop_a.
-template <int TI, int RW>
+template <int TI, int RW, int RM>
 __device__ __forceinline__ void fused_loop_a(const FusedCtx& c, const BwdUnit& u, const FusedTask* __restrict__ ft,
                                              float2* __restrict__ dst) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
@@ -1348,7 +1565,7 @@ __device__ __forceinline__ void fused_loop_a(const FusedCtx& c, const BwdUnit& u
     }
     fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
         const BwdGeom q{ft_l(t), u.l1, ft_l2(t), u.rows, ft_tau2(t)};
-        bwd_accum<1, TI, RW>(q, cgp, reinterpret_cast<const float2*>(c.tile), f2, c.tid, ax, ay);
+        bwd_accum<1, TI, RW, RM>(q, cgp, reinterpret_cast<const float2*>(c.tile), f2, c.tid, ax, ay);
         if (ft_last(t)) {
 #pragma unroll
             for (int i = 0; i < TI; ++i)
@@ -1447,8 +1664,8 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
     // the first stage waits for these copies
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
-#define CGNET_LOOP_A(TI_, RW_) fused_loop_a<TI_, RW_>(c, u, ft, dst)
-        CGNET_BWD_SWITCH(u.TI, u.RW, CGNET_LOOP_A)
+#define CGNET_LOOP_A(TI_, RW_, RM_) fused_loop_a<TI_, RW_, RM_>(c, u, ft, dst)
+        CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
         fused_loop_b(c, u, ft, wave - u.nA, kHybWaves - u.nA, part2 + (size_t)b * P2);
@@ -1794,7 +2011,17 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     // One launch has one LDS size, and the largest task's would set the occupancy of all: the tasks are
     // grouped by the number of work-groups per compute unit their own LDS need allows (at most four, the
     // register limit), largest need first, and every class gets a launch of its own.
-    auto fwd_class = [](const CgTask& t) { return (int)std::max<size_t>(1, std::min<size_t>(4, kMaxLds / align_up(fwd_task_lds(t), 16))); };
+    // Product on the matrix cores when every channel count fills a good part of a 16 x 16 tile
+    // (CGNET_FWD_MM=0 keeps the vector-ALU kernel).
+    p->fwd_mm = true;
+    for (int l = 0; l < n1; ++l)
+        if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) p->fwd_mm = false;
+    for (const CgTask& t : p->fwd_tasks)
+        if (t.rows > 16) p->fwd_mm = false;
+    if (const char* e = getenv("CGNET_FWD_MM"); e && e[0] == '0') p->fwd_mm = false;
+    const bool fwd_mm = p->fwd_mm;
+    auto fwd_need = [fwd_mm](const CgTask& t) { return align_up(fwd_mm ? fwd_task_lds_mm(t) : fwd_task_lds(t), 16); };
+    auto fwd_class = [&](const CgTask& t) { return (int)std::max<size_t>(1, std::min<size_t>(4, kMaxLds / fwd_need(t))); };
     std::stable_sort(p->fwd_tasks.begin(), p->fwd_tasks.end(),
                      [&](const CgTask& a, const CgTask& b) { return fwd_class(a) < fwd_class(b); });
     p->fwd_class_begin.clear();
@@ -1804,12 +2031,12 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             p->fwd_class_begin.push_back((int)k);
             p->fwd_class_lds.push_back(0);
         }
-        p->fwd_class_lds.back() = std::max(p->fwd_class_lds.back(), align_up(fwd_task_lds(p->fwd_tasks[k]), 16));
+        p->fwd_class_lds.back() = std::max(p->fwd_class_lds.back(), fwd_need(p->fwd_tasks[k]));
     }
     p->fwd_class_begin.push_back((int)p->fwd_tasks.size());
     size_t fl = 0, bl = 0;
     for (const CgTask& t : p->fwd_tasks) {
-        fl = std::max(fl, fwd_task_lds(t));
+        fl = std::max(fl, fwd_need(t));
         CGNET_REQUIRE(2 * fwd_frag_lds(t) <= kMaxUnitLds, CGNET_ERR_UNSUPPORTED,
                       "fragment slabs of %zu bytes exceed the LDS staging window", 2 * fwd_frag_lds(t));
     }
@@ -1877,6 +2104,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         for (int l = 0; l < n1; ++l)
             if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) hybrid = false;
         if (const char* e = getenv("CGNET_BWD_HYBRID"); e && e[0] == '0') hybrid = false;
+        bool use_rm = true;      // CGNET_BWD_MSPLIT=0: lanes of an item split only the reduced channels
+        if (const char* e = getenv("CGNET_BWD_MSPLIT"); e && e[0] == '0') use_rm = false;
         if (attempt == 0 && !hybrid) continue;
         const long long tile_limit = hybrid ? kHybTileBytes : kBwdTileBytes;
         int f1cap = 0, f2cap = 0, cgcap = 0, tcap = 0;
@@ -1894,7 +2123,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             });
             const int tau1 = h_t_F[l1], M1 = 2 * l1 + 1;
             const int nt = (int)tri.size();
-            struct Choice { double total = -1; int rows = 0, nA = 0, TI = 0, RW = 0; std::vector<int> bTI, bRW; std::vector<double> tcost; };
+            struct Choice { double total = -1; int rows = 0, nA = 0, TI = 0, RW = 0, RM = 1; std::vector<int> bTI, bRW; std::vector<double> tcost; };
             Choice best;
             int prev_rows = -1;
             for (int nchunks = 1; nchunks <= tau1; ++nchunks) {
@@ -1937,26 +2166,33 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     int max_tau2 = 1;
                     for (int i : tri) max_tau2 = std::max(max_tau2, h_t_F[tl2[i]]);
                     for (int ti = 1; ti <= kBwdMaxTI; ++ti)
-                        for (int rw = 1; rw <= 16; rw *= 2) {
-                            if (rw > 1 && rw / 2 >= max_tau2) continue;
-                            const int items = ((rows_c + ti - 1) / ti) * ((M1 + 1) / 2);
-                            if (items * rw > lanesA) continue;
-                            double total = 0;
-                            std::vector<double> tcost(nt);
-                            for (int k = 0; k < nt; ++k) {
-                                const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
-                                const double scaleA = hybrid ? kHybSlot1Scale : 1.0;
-                                const double cA = scaleA * ((tau2 + rw - 1) / rw) * (double)M2 * (8.0 * ti + 14.0);
-                                const double stage = 12.0 * rows_c * tau2 * (2 * tl[tri[k]] + 4) / kThreads + 200.0;
-                                tcost[k] = std::max(cA, costB[k]) + stage;
-                                total += tcost[k];
+                        for (int rw = 1; rw <= 16; rw *= 2)
+                            for (int rm = 1; rm <= 2; ++rm) {
+                                // rm = 2: half of the lanes of an item take the second half of the reduced m range
+                                if (rm == 2 && (rw < 4 || ti < 2 || !use_rm)) continue;
+                                const int rc = rw / rm;
+                                if (rc > 1 && rc / 2 >= max_tau2) continue;
+                                const int items = ((rows_c + ti - 1) / ti) * ((M1 + 1) / 2);
+                                if (items * rw > lanesA) continue;
+                                double total = 0;
+                                std::vector<double> tcost(nt);
+                                for (int k = 0; k < nt; ++k) {
+                                    const int tau2 = h_t_F[tl2[tri[k]]], M2 = 2 * tl2[tri[k]] + 1;
+                                    const double scaleA = hybrid ? kHybSlot1Scale : 1.0;
+                                    // steps of the busiest lane: its channels x its part of the m range (in step pairs)
+                                    const double msteps = rm == 1 ? (double)M2 : 2.0 * ((M2 / 2 + 2) / 2) + 1.0;
+                                    const double cA = scaleA * ((tau2 + rc - 1) / rc) * msteps * (8.0 * ti + 14.0);
+                                    const double stage = 12.0 * rows_c * tau2 * (2 * tl[tri[k]] + 4) / kThreads + 200.0;
+                                    tcost[k] = std::max(cA, costB[k]) + stage;
+                                    total += tcost[k];
+                                }
+                                total *= real_chunks;
+                                if (best.total < 0 || total < best.total) {
+                                    best.total = total; best.rows = rows_c; best.nA = nA; best.TI = ti; best.RW = rw;
+                                    best.RM = rm;
+                                    best.bTI = bTI; best.bRW = bRW; best.tcost = tcost;
+                                }
                             }
-                            total *= real_chunks;
-                            if (best.total < 0 || total < best.total) {
-                                best.total = total; best.rows = rows_c; best.nA = nA; best.TI = ti; best.RW = rw;
-                                best.bTI = bTI; best.bRW = bRW; best.tcost = tcost;
-                            }
-                        }
                 }
             }
             if (best.total < 0) { ok = false; break; }
@@ -1967,7 +2203,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 u.offF1 = p->cumF[l1] + r0 * M1;
                 u.offF1p = cumFp[l1] + r0 * (M1 + 1);
                 u.task_begin = (int)p->bwd_utasks.size();
-                u.nA = best.nA; u.TI = best.TI; u.RW = best.RW;
+                u.nA = best.nA; u.TI = best.TI; u.RW = best.RW; u.RM = best.RM;
                 u.p1off = -1;
                 f1cap = std::max(f1cap, (int)align_up((size_t)8 * u.rows * (M1 + 1), 16));
                 for (int k = 0; k < nt; ++k) {
@@ -2081,8 +2317,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 for (const BwdUnit& u : p->bwd_units) {
                     const BwdUTask& t0 = p->bwd_utasks[u.task_begin];
                     const BwdUTask& t1 = p->bwd_utasks[u.task_end - 1];
-                    fprintf(stderr, "[cgnet]   l1=%d rows=%d tasks=%d nA=%d A(TI=%d,RW=%d) B first(TI=%d,RW=%d) last(TI=%d,RW=%d)\n",
-                            u.l1, u.rows, u.task_end - u.task_begin, u.nA, u.TI, u.RW, t0.TI, t0.RW, t1.TI, t1.RW);
+                    fprintf(stderr, "[cgnet]   l1=%d rows=%d tasks=%d nA=%d A(TI=%d,RW=%d,RM=%d) B first(TI=%d,RW=%d) last(TI=%d,RW=%d)\n",
+                            u.l1, u.rows, u.task_end - u.task_begin, u.nA, u.TI, u.RW, u.RM, t0.TI, t0.RW, t1.TI, t1.RW);
                 }
             }
             p->bwd_fast_lds = align_up(lds_max, 16);
@@ -2122,7 +2358,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                                        p->bwd_fast_lds))
             return rc;
     }
-    if (int rc = raise_dynamic_lds((const void*)cg_forward_kernel, p->fwd_lds)) return rc;
+    if (int rc = raise_dynamic_lds(p->fwd_mm ? (const void*)cg_forward_mm_kernel : (const void*)cg_forward_kernel, p->fwd_lds)) return rc;
     if (int rc = raise_dynamic_lds((const void*)cg_backward_kernel, p->bwd_lds)) return rc;
     *plan = guard.release();
     return CGNET_OK;
@@ -2167,9 +2403,15 @@ static int launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF,
                   "%d tasks x %d sample groups exceed the grid limit", ntasks, ngroups);
     for (size_t k = 0; k + 1 < p->fwd_class_begin.size(); ++k) {
         const int t0 = p->fwd_class_begin[k], nt = p->fwd_class_begin[k + 1] - t0;
-        CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(nt * ngroups)), dim3(kThreads), p->fwd_class_lds[k], s,
-                           (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
-                           p->sumT);
+        if (p->fwd_mm) {
+            CGNET_LAUNCH(cg_forward_mm_kernel, dim3((unsigned)(nt * ngroups)), dim3(kFwdMmThreads), p->fwd_class_lds[k], s,
+                         (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
+                         p->sumT, (int)p->fwd_class_lds[k]);
+        } else {
+            CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(nt * ngroups)), dim3(kThreads), p->fwd_class_lds[k], s,
+                         (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
+                         p->sumT);
+        }
         CGNET_HIP(hipGetLastError());
     }
     return CGNET_OK;
