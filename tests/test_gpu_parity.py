@@ -139,6 +139,30 @@ CG_CASES = [
 ]
 
 
+def edge_pairs(lmax):
+    """A short custom triple list that reaches the highest degrees in every slot: per output degree l the pairs
+    (l, 0) and (lmax, lmax - l), and (lmax, lmax) for l = 0 and l = lmax (the largest coefficient table)."""
+    pairs = []
+    for l in range(lmax + 1):
+        here = {(l, 0), (lmax, lmax - l)}
+        if l in (0, lmax):
+            here.add((lmax, lmax))
+        pairs.append(sorted(here))
+    return pairs
+
+
+# Degrees above 23 (the library accepts lmax up to sparse_maxL() = 47): few triples and channels, so that the CPU
+# oracle stays within seconds.  They reach the tables of up to 95 x 95 coefficients and the backward kernels that
+# take over where the matrix-core unit kernel stops.
+HIGH_DEGREE_CG_CASES = [
+    (24, [2] * 25, 2, edge_pairs(24)),
+    (24, [1, 2] * 12 + [1], 1, "debug"),
+    (47, [1, 2] * 24, 1, edge_pairs(47)),
+    (47, [2] * 48, 2, "debug"),
+    (30, [9] * 31, 1, edge_pairs(30)),                    # channel counts in 8..16 above the matrix-core kernels' lmax
+]
+
+
 def cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64=None, dtype=F64):
     x = x64.to(dtype).clone().requires_grad_(True)
     y = OL.join_straight(OL.cg_product(x, lmax, codes, taus))
@@ -146,6 +170,12 @@ def cg_oracle_fwd_bwd(lmax, taus, codes, x64, gy64=None, dtype=F64):
         return y.detach(), None
     (gx,) = torch.autograd.grad(y, x, gy64.to(dtype))
     return y.detach(), gx
+
+
+@pytest.mark.parametrize("lmax,taus,bsz,mode", HIGH_DEGREE_CG_CASES,
+                         ids=["L24-edge", "L24-debug", "L47-edge", "L47-debug", "L30-edge-tau9"])
+def test_cg_forward_backward_high_degrees(dev, lmax, taus, bsz, mode):
+    test_cg_forward_backward(dev, lmax, taus, bsz, mode)
 
 
 @pytest.mark.parametrize("lmax,taus,bsz,mode", CG_CASES)
@@ -293,6 +323,12 @@ WMM_CASES = [
     (2, [1, 1, 1], [1, 1, 1], 1, True, True),
     (11, [300, 500, 700, 900, 1100, 1200, 1300, 1300, 1300, 1250, 1180, 1050], [12] * 12, 9, True, True),
     (20, [64] * 21, [16] * 21, 3, True, True),                    # 41 complex columns per sample
+    # degrees above 23: 49 .. 95 complex columns per sample (four to six column tiles in the matrix-core kernels)
+    (24, [9 + (l % 12) for l in range(25)], [3] * 25, 3, True, True),
+    (24, [9 + (l % 12) for l in range(25)], [17] * 25, 3, True, True),
+    (47, [9 + (l % 12) for l in range(48)], [3 if l % 2 else 17 for l in range(48)], 3, True, True),
+    (47, [20 - (l % 12) for l in range(48)], [12] * 48, 2, False, True),
+    (36, [40] * 37, [16] * 37, 5, True, False),
 ]
 
 
@@ -484,6 +520,18 @@ def test_layer_config5_shape(dev):
     mod, ora, twin, w64 = build_layer_pair(dev, lmax, tau, tau, False, True, seed=20)
     x64 = rand_straight(tau, 1, seed=22)
     go64 = randn32((1, 16 * 441, 2), torch.Generator().manual_seed(24))
+    check_layer_step(dev, mod, ora, twin, w64, x64, go64)
+
+
+def test_layer_high_degree(dev):
+    """One training step of a layer at lmax = 24 (spanning-tree triples, one channel in, two out, B = 2): the product,
+    the statistics and the mixing kernels with 49 complex columns per sample."""
+    lmax = 24
+    tin, tout = [1] * 25, [2] * 25
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, True, True, seed=24)
+    x64 = rand_straight(tin, 2, seed=26)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go64 = randn32((2, n_o, 2), torch.Generator().manual_seed(28))
     check_layer_step(dev, mod, ora, twin, w64, x64, go64)
 
 
