@@ -412,18 +412,23 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
 // the middle outwards, and writes its 16 x 16 results into the output tile; the tile then leaves as in the
 // vector-ALU kernel.  Used when every channel count is in 8..16.
 constexpr int kFwdMmPad = 32;     // bytes before / between / behind the fragment buffers
+constexpr size_t kFwdMmStatsLds = 8 * 256 * sizeof(double);   // eight waves x four values x 64 lanes
 
 __host__ __device__ inline size_t fwd_task_lds_mm(const CgTask& t) {
     const size_t M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
-    return kFwdMmPad + 2 * (fwd_frag_lds(t) + kFwdMmPad) + ((8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15) +
-           ((4 * M * (M2 + 3) + 15) & ~(size_t)15);
+    const size_t need = kFwdMmPad + 2 * (fwd_frag_lds(t) + kFwdMmPad) +
+                        ((8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15) + ((4 * M * (M2 + 3) + 15) & ~(size_t)15);
+    return need > kFwdMmStatsLds ? need : kFwdMmStatsLds;     // the statistics' final reduction runs through LDS
 }
 
 // One sample of a task: the waves take the values of m in turn (from the middle outwards, so that every wave gets
 // long and short ones); for one m the accumulator D[t1][t2] gathers the steps of four m2.
+// STATS: the lane also adds |z| and |z|^2 of its four results (channels (4 kk + v, i)) to its own sums.
+template <bool STATS>
 __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __restrict__ cg, int P,
                                               const float2* __restrict__ f1, const float2* __restrict__ f2,
-                                              float2* __restrict__ out, int wave, int nwaves, int lane) {
+                                              float2* __restrict__ out, int wave, int nwaves, int lane,
+                                              double (&s1)[4], double (&s2)[4]) {
     const int l = t.l, l1 = t.l1, l2 = t.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = t.rows, tau2 = t.tau2;
@@ -462,12 +467,22 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
             for (int v = 0; v < 4; ++v)
                 if (4 * kk + v < rows) o[v * tau2 * M] = make_float2(dre[v], dim[v]);
         }
+        if (STATS) {
+            // both sums run over the same rounded |z| in double (see cg_forward_kernel); lanes past the task's
+            // channels add up values nobody reads
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const double r = (double)sqrt_hw(fmaf(dre[v], dre[v], dim[v] * dim[v]));
+                s1[v] += r;
+                s2[v] = fma(r, r, s2[v]);
+            }
+        }
     }
 }
 
 constexpr int kFwdMmThreads = 512;
 
-__global__ void __launch_bounds__(kFwdMmThreads)
+__global__ void __launch_bounds__(kFwdMmThreads, 8)    // 64 registers: four work-groups per compute unit
 cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const float* __restrict__ CG,
                      const CgTask* __restrict__ tasks, int nF, int nFF, int B, int samples_per_group,
                      double* __restrict__ stats_part, int sumT, int lds_bytes) {
@@ -501,7 +516,7 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
         dma16<kFwdMmThreads>(Fb + t.offF2, d2, n2 >> 1, tid);
         if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
     };
-    double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};
+    double s1[4] = {0., 0., 0., 0.}, s2[4] = {0., 0., 0., 0.};   // of the lane's channels, over its m and all samples
     const int b0 = group * samples_per_group;
     const int b1 = min(B, b0 + samples_per_group);
     if (b0 < b1) issue(b0, 0);
@@ -518,7 +533,8 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
         const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
         const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
 #ifndef CGNET_TEST_FWD_NOCOMPUTE
-        fwd_mm_sample(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane);
+        if (stats_part) fwd_mm_sample<true>(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane, s1, s2);
+        else fwd_mm_sample<false>(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane, s1, s2);
 #endif
         __syncthreads();
         // tile -> FF with 16-byte stores from the first 16-byte boundary on
@@ -534,33 +550,26 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
 #endif
         if (tid == 0 && head) dst[0] = out[0];
         if (tid == 1 && ((nout - head) & 1)) dst[nout - 1] = out[nout - 1];
-        if (stats_part) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int ch = tid + kFwdMmThreads * k;
-                if (ch < nch) {
-                    // both sums run over the same rounded |z| in double (see cg_forward_kernel)
-                    double a = s1[k], q = s2[k];
-                    for (int mm = 0; mm < M; ++mm) {
-                        const float2 z = out[ch * M + mm];
-                        const double r = (double)sqrt_hw(fmaf(z.x, z.x, z.y * z.y));
-                        a += r;
-                        q = fma(r, r, q);
-                    }
-                    s1[k] = a;
-                    s2[k] = q;
-                }
-            }
-        }
     }
     if (stats_part) {
+        // The eight waves hold partial sums of the same channels (each over its own m).  They go through LDS
+        // (everything else in it is no longer needed) in two rounds of four values per lane, and one thread
+        // per channel adds the waves in order.
+        double* red = reinterpret_cast<double*>(smem);            // [wave][value 0..3][lane]
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int ch = tid + kFwdMmThreads * k;
-            if (ch < nch) {
-                double* p = stats_part + ((size_t)group * sumT + t.chan0 + ch) * 2;
-                p[0] = s1[k];
-                p[1] = s2[k];
+        for (int round = 0; round < 2; ++round) {
+            __syncthreads();                                       // the last tile has left / round 0 has been read
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[(wave * 4 + v) * 64 + lane] = round == 0 ? s1[v] : s2[v];
+            __syncthreads();
+            // thread -> channel (row r, column c) of the task; its value lies at lane (r / 4) * 16 + c, slot r % 4
+            for (int ch = tid; ch < nch; ch += kFwdMmThreads) {
+                const int r = ch / t.tau2, c = ch - r * t.tau2;
+                const int src = (r & 3) * 64 + (r >> 2) * 16 + c;
+                double sum = 0.;
+#pragma unroll
+                for (int w = 0; w < kFwdMmThreads / 64; ++w) sum += red[w * 256 + src];
+                stats_part[((size_t)group * sumT + t.chan0 + ch) * 2 + round] = sum;
             }
         }
     }
