@@ -408,9 +408,9 @@ cg_forward_kernel(const float2* __restrict__ F, float2* __restrict__ FF, const f
 // and step); the right operand is read as it lies in the staged l2 slab.  No masking: the table is staged with three
 // zeros behind every row, and holds zeros where m - m2 is no valid m1 (every table this library fills does), so the
 // steps past the last valid m2 multiply whatever finite fragment entries lie next to the rows by zero (LDS is
-// cleared once, the slabs have 32 spare bytes on either side).  Every wave takes every fourth m, numbered from
-// the middle outwards, and writes its 16 x 16 results into the output tile; the tile then leaves as in the
-// vector-ALU kernel.  Used when every channel count is in 8..16.
+// cleared once, the slabs have 32 spare bytes on either side).  The eight waves take the values of m in turn,
+// numbered from the middle outwards, and write their 16 x 16 results into the output tile; the tile then leaves as
+// in the vector-ALU kernel.  Used when every channel count is in 8..16.
 constexpr int kFwdMmPad = 32;     // bytes before / between / behind the fragment buffers
 constexpr size_t kFwdMmStatsLds = 8 * 256 * sizeof(double);   // eight waves x four values x 64 lanes
 
@@ -532,22 +532,18 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
         if (b + 1 < b1) issue(b + 1, par ^ 1);
         const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
         const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
-#ifndef CGNET_TEST_FWD_NOCOMPUTE
         if (stats_part) fwd_mm_sample<true>(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane, s1, s2);
         else fwd_mm_sample<false>(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane, s1, s2);
-#endif
         __syncthreads();
         // tile -> FF with 16-byte stores from the first 16-byte boundary on
         float2* dst = FF + (size_t)b * nFF + t.offFF;
         const int head = min(nout, (int)((reinterpret_cast<uintptr_t>(dst) >> 3) & 1));
         const int npair = (nout - head) >> 1;
         float4* dst4 = reinterpret_cast<float4*>(dst + head);
-#ifndef CGNET_TEST_FWD_NOSTORE
         for (int e = tid; e < npair; e += kFwdMmThreads) {
             const float2 u = out[head + 2 * e], v = out[head + 2 * e + 1];
             stream_store16(dst4 + e, u.x, u.y, v.x, v.y);
         }
-#endif
         if (tid == 0 && head) dst[0] = out[0];
         if (tid == 1 && ((nout - head) & 1)) dst[nout - 1] = out[nout - 1];
     }
@@ -1108,9 +1104,7 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         const float2 *g, *f2;
         bwd_stage<NT>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
-#ifndef CGNET_TEST_NOSLOT1
         bwd_accum<1, TI, RW, RM>(q, cgp, g, f2, c.rtid, ax, ay);
-#endif
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
 #pragma unroll
@@ -1340,14 +1334,12 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
     if (cur.l2 <= 7) { CGNET_MM_NT(NK_, 1) }                            \
     else if (cur.l2 <= 15) { CGNET_MM_NT(NK_, 2) }                      \
     else { CGNET_MM_NT(NK_, 3) }
-#ifndef CGNET_TEST_NOSLOT2
         switch ((u.rows + 3) >> 2) {
             case 1: CGNET_MM(1) break;
             case 2: CGNET_MM(2) break;
             case 3: CGNET_MM(3) break;
             default: CGNET_MM(4) break;
         }
-#endif
 #undef CGNET_MM_NT
 #undef CGNET_MM_CALL
 #undef CGNET_MM
@@ -1545,12 +1537,8 @@ __device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTa
                 dma16<kHybThreads>(c.Fp + nxt.offF2p, c.f2 + (f2par ^ 1) * c.f2cap,
                                    (ft_tau2(nxt) * (2 * ft_l2(nxt) + 2)) >> 1, c.tid);
         }
-#ifndef CGNET_TEST_NOGEN
         gen_phase(cur, c.al, c.bl, c.tile, c.wave, c.lane);
-#endif
-#ifndef CGNET_TEST_NOBAR2
         lds_barrier();         // the tile is complete; the operand buffers are free
-#endif
         if (more) {
             dma16<kHybThreads>(c.Ag + nxt.aoff, c.al, nxt.chunks & 0xffff, c.tid);
             dma16<kHybThreads>(c.Bg + nxt.boff, c.bl, nxt.chunks >> 16, c.tid);
@@ -1801,6 +1789,10 @@ partial_sum_kernel(const float2* __restrict__ part, float2* __restrict__ out, si
 __global__ void __launch_bounds__(256) fill_zero_f64_kernel(double* p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0.;
+}
+
+__global__ void __launch_bounds__(256) fill_zero_f32_kernel(float* p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
 // ------------------------------------------------------------------------------------- host
@@ -2454,7 +2446,10 @@ extern "C" int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float
     CGNET_REQUIRE(d_sums, CGNET_ERR_ARG, "d_sums is NULL");
     hipStream_t s = (hipStream_t)stream;
     if (B == 0 || plan->nFF == 0) {
-        CGNET_HIP(hipMemsetAsync(d_sums, 0, sizeof(double) * 2 * plan->sumT, s));
+        // a fill kernel, not hipMemsetAsync: the call may be recorded into a graph
+        const int n2 = 2 * plan->sumT;
+        CGNET_LAUNCH(fill_zero_f64_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s, d_sums, n2);
+        CGNET_HIP(hipGetLastError());
         return CGNET_OK;
     }
     CGNET_REQUIRE(d_F && d_FF && d_CG, CGNET_ERR_ARG, "null device pointer");
@@ -2531,7 +2526,11 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
     hipStream_t s = (hipStream_t)stream;
     const int ng_max = (int)plan->bwd_group_begin.size() - 1;
     if (ng_max <= 0 || plan->bwd_tasks.empty()) {
-        CGNET_HIP(hipMemsetAsync(d_gF, 0, sizeof(float) * 2 * (size_t)plan->nF * B, s));
+        // no triple contributes: the gradient is zero (a fill kernel, not hipMemsetAsync: the call may be recorded
+        // into a graph)
+        const size_t nf = 2 * (size_t)plan->nF * B;
+        CGNET_LAUNCH(fill_zero_f32_kernel, dim3((unsigned)std::min<size_t>((nf + 255) / 256, 4096)), dim3(256), 0, s, d_gF, nf);
+        CGNET_HIP(hipGetLastError());
         return CGNET_OK;
     }
     CGNET_REQUIRE(d_F && d_gFF && d_CG, CGNET_ERR_ARG, "null device pointer");

@@ -932,6 +932,24 @@ def test_errors(dev):
     assert y.shape[0] == 0
 
 
+def test_cg_without_contributing_triples(dev):
+    """A triple list none of whose triples has channels in both slots: the product is empty, the statistics and the
+    input gradient are zero (written by fill kernels, so that the calls can be recorded into a graph)."""
+    from cgnet_amd import CG_layers
+    taus = [2, 0]
+    mod = CG_layers.CG_woFilter_cuda(1, taus, lll_mode=[[(1, 1)], [(1, 0)]], device=dev)
+    plan = mod.native_plan()
+    assert plan.nFF == 0 and plan.nF == 2
+    bsz = 3
+    x = torch.randn(bsz, 2, 2, device=dev)
+    gF = torch.full((bsz, 2, 2), 7.0, device=dev)
+    empty = torch.empty(bsz, 0, 2, device=dev)
+    plan.backward(x, gF, empty, mod.CGspace, bsz)
+    assert torch.equal(gF, torch.zeros_like(gF))
+    y = mod(x, straight_output=True)
+    assert y.shape == (bsz, 0, 2)
+
+
 # ------------------------------------------------------------------------------- timing hooks
 def test_kernel_timing_hooks(dev):
     """Every launch is bracketed when timing is on; cgnet_profile_select narrows it to one kernel."""
