@@ -103,6 +103,7 @@ struct cgnet_cg_plan {
     int* d_bwd_group_table = nullptr;
     size_t fwd_lds = 0, bwd_lds = 0;
     bool fwd_mm = false;                         // the forward runs cg_forward_mm_kernel (product on the matrix cores)
+    bool bwd_general_ok = true;                  // cg_backward_kernel's LDS need fits (else only the unit kernels serve)
     std::vector<int> fwd_class_begin;            // forward tasks by LDS class: class k = tasks [begin[k], begin[k+1])
     std::vector<size_t> fwd_class_lds;           // LDS bytes of a work-group of class k
     int bwd_threads = 256;                       // work-group size of the backward kernel
@@ -140,6 +141,8 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kFwdTileBytes = 32 * 1024;
+constexpr int kFwdMmTileBytes = 128 * 1024;      // matrix-core forward: 16 x 16 channels x 95 values of m = 190 KB at
+                                                 // most, the largest that leaves room for the operands
 constexpr int kBwdTileBytes = 14 * 1024;
 constexpr int kMaxTileChannels = 4 * kThreads;   // statistics: at most four channels per thread
 constexpr int kMaxBwdGroups = 32;
@@ -1919,7 +1922,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     p->nFF = p->cumFF[n1];
     p->sumT = p->cumT[n1];
 
-    auto build = [&](int tile_bytes, std::vector<CgTask>* out, int pad = 0) -> int {
+    auto build = [&](int tile_bytes, std::vector<CgTask>* out, int pad = 0, bool mm = false) -> int {
         for (int i = 0; i < nllls; ++i) {
             const int l = tl[i], l1 = tl1[i], l2 = tl2[i];
             const int tau1 = h_t_F[l1], tau2 = h_t_F[l2];
@@ -1928,6 +1931,13 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             const long long row_bytes = 8LL * tau2 * (M + pad);
             int max_rows = (int)std::min<long long>(tau1, std::max<long long>(1, tile_bytes / row_bytes));
             max_rows = std::max(1, std::min(max_rows, kMaxTileChannels / tau2));
+            if (mm) {
+                // the whole work-group (tile, two pairs of fragment slabs, padded table) has to fit the LDS
+                CgTask probe;
+                probe.l = l; probe.l1 = l1; probe.l2 = l2; probe.tau1 = tau1; probe.tau2 = tau2;
+                for (probe.rows = max_rows; probe.rows > 1 && fwd_task_lds_mm(probe) > kMaxLds; --probe.rows) {}
+                max_rows = probe.rows;
+            }
             const int nchunks = (tau1 + max_rows - 1) / max_rows;
             const int rows_per = (tau1 + nchunks - 1) / nchunks;
             for (int r0 = 0; r0 < tau1; r0 += rows_per) {
@@ -1965,7 +1975,14 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         }
         return 0;
     };
-    build(kFwdTileBytes, &p->fwd_tasks);
+    // Product on the matrix cores when every channel count fills a good part of a 16 x 16 tile (CGNET_FWD_MM=0
+    // keeps the vector-ALU kernel).  Its tasks then take all rows of a triple -- a row block of six of sixteen
+    // rows, which the 32 KB limit gives at 41 values of m, fills the matrix tiles to 37 % -- up to kFwdMmTileBytes.
+    p->fwd_mm = true;
+    for (int l = 0; l < n1; ++l)
+        if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) p->fwd_mm = false;
+    if (const char* e = getenv("CGNET_FWD_MM"); e && e[0] == '0') p->fwd_mm = false;
+    build(p->fwd_mm ? kFwdMmTileBytes : kFwdTileBytes, &p->fwd_tasks, 0, p->fwd_mm);
     p->bwd_tasks.clear();
     build(kBwdTileBytes, &p->bwd_tasks, kPadLo + kPadHi);
     // Backward tiling.  Per slot a thread owns TI output channels x 2 m and RW lanes split the
@@ -2012,14 +2029,6 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     // One launch has one LDS size, and the largest task's would set the occupancy of all: the tasks are
     // grouped by the number of work-groups per compute unit their own LDS need allows (at most four, the
     // register limit), largest need first, and every class gets a launch of its own.
-    // Product on the matrix cores when every channel count fills a good part of a 16 x 16 tile
-    // (CGNET_FWD_MM=0 keeps the vector-ALU kernel).
-    p->fwd_mm = true;
-    for (int l = 0; l < n1; ++l)
-        if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) p->fwd_mm = false;
-    for (const CgTask& t : p->fwd_tasks)
-        if (t.rows > 16) p->fwd_mm = false;
-    if (const char* e = getenv("CGNET_FWD_MM"); e && e[0] == '0') p->fwd_mm = false;
     const bool fwd_mm = p->fwd_mm;
     auto fwd_need = [fwd_mm](const CgTask& t) { return align_up(fwd_mm ? fwd_task_lds_mm(t) : fwd_task_lds(t), 16); };
     auto fwd_class = [&](const CgTask& t) { return (int)std::max<size_t>(1, std::min<size_t>(4, kMaxLds / fwd_need(t))); };
@@ -2046,8 +2055,10 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
     p->bwd_lds = align_up(bl, 16) + 8 * (size_t)p->nF;
     CGNET_REQUIRE(p->fwd_lds <= kMaxLds, CGNET_ERR_UNSUPPORTED,
                   "a single output row needs %zu bytes of LDS (limit %zu)", p->fwd_lds, kMaxLds);
-    CGNET_REQUIRE(p->bwd_lds <= kMaxLds, CGNET_ERR_UNSUPPORTED,
-                  "backward needs %zu bytes of LDS (limit %zu): too many input channels", p->bwd_lds, kMaxLds);
+    // The LDS-accumulator backward keeps a sample's whole input gradient in LDS.  Where that does not fit, the
+    // backward depends on the unit kernels below; where they do not fit either, the plan serves the forward only and
+    // cgnet_sparse_backward reports the shape as unsupported.
+    p->bwd_general_ok = p->bwd_lds <= kMaxLds;
 
     // backward groups: contiguous task ranges of roughly equal cost, at most kMaxBwdGroups
     {
@@ -2360,7 +2371,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             return rc;
     }
     if (int rc = raise_dynamic_lds(p->fwd_mm ? (const void*)cg_forward_mm_kernel : (const void*)cg_forward_kernel, p->fwd_lds)) return rc;
-    if (int rc = raise_dynamic_lds((const void*)cg_backward_kernel, p->bwd_lds)) return rc;
+    if (p->bwd_general_ok)
+        if (int rc = raise_dynamic_lds((const void*)cg_backward_kernel, p->bwd_lds)) return rc;
     *plan = guard.release();
     return CGNET_OK;
 }
@@ -2570,6 +2582,9 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
         CGNET_HIP(hipGetLastError());
         return CGNET_OK;
     }
+    CGNET_REQUIRE(plan->bwd_general_ok, CGNET_ERR_UNSUPPORTED,
+                  "backward needs %zu bytes of LDS (limit %zu): too many input channels for this lmax; the plan serves "
+                  "the forward only", plan->bwd_lds, kMaxLds);
     const int* d_gb = plan->d_bwd_group_table + plan->bwd_group_table_off[ng];
     float2* dst = ng > 1 ? (float2*)d_workspace : (float2*)d_gF;
     CGNET_LAUNCH(cg_backward_kernel, dim3(ng, B), dim3(plan->bwd_threads), plan->bwd_lds, s,

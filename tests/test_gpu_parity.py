@@ -178,6 +178,24 @@ def test_cg_forward_backward_high_degrees(dev, lmax, taus, bsz, mode):
     test_cg_forward_backward(dev, lmax, taus, bsz, mode)
 
 
+def test_cg_forward_only_shape(dev):
+    """lmax = 47 with 16 channels per degree: the forward runs (matrix cores, row blocks cut so that a work-group
+    fits the LDS); no backward kernel can hold the shape, and the backward call says so instead of the plan failing."""
+    from cgnet_amd import CG_layers, _lib
+    lmax, taus, bsz = 47, [16] * 48, 1
+    pairs = edge_pairs(lmax)
+    codes = make_codes(lmax, pairs)
+    x64 = rand_straight(taus, bsz, seed=47)
+    mod = CG_layers.CG_woFilter_cuda(lmax, taus, lll_mode=pairs, device=dev)
+    want_y, _ = cg_oracle_fwd_bwd(lmax, taus, codes, x64)
+    twin_y, _ = cg_oracle_fwd_bwd(lmax, taus, codes, x64, dtype=F32)
+    x = x64.float().to(dev).requires_grad_(True)
+    y = mod(x, straight_output=True)
+    assert_close(y, want_y, "CG forward, lmax 47, 16 channels", twin_y)
+    with pytest.raises(_lib.CgnetError, match="forward only"):
+        y.backward(torch.ones_like(y))
+
+
 @pytest.mark.parametrize("lmax,taus,bsz,mode", CG_CASES)
 def test_cg_forward_backward(dev, lmax, taus, bsz, mode):
     from cgnet_amd import CG_layers
