@@ -58,8 +58,10 @@ def assert_close(got, ref, what, twin=None, rtol=RTOL, atol=ATOL):
     err = (got - ref).abs()
     err_twin = float((_flat(twin) - ref).abs().max()) if twin is not None else 0.0
     bound = torch.clamp(strict, min=TWIN_FACTOR * err_twin)
+    rms = lambda e: float(torch.sqrt(torch.mean(e * e)))
     rec = {"test": os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0], "what": what, "n": ref.numel(),
            "max_ref": float(ref.abs().max()), "err_gpu": float(err.max()), "err_cpu32": err_twin if twin is not None else None,
+           "rms_gpu": rms(err), "rms_cpu32": rms(_flat(twin) - ref) if twin is not None else None,
            "strict_violations_gpu": int((err > strict).sum()),
            "strict_violations_cpu32": int(((_flat(twin) - ref).abs() > strict).sum()) if twin is not None else None}
     print("[parity] %-28s max|ref| %.3e  err_gpu %.3e  err_cpu32 %s  outside strict bar: gpu %d cpu32 %s of %d"
