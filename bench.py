@@ -62,6 +62,27 @@ def profiled_traffic():
     return table, "%s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; measured at %s, not in this run)" % (TRAFFIC_PROFILE, rev)
 
 
+SQ_PROFILE = os.path.join("profiles", "cg_layer_L11_tau12_B100_sq_counters_pmc.txt")
+
+
+def profiled_issue(kernel, avg_launch_ms):
+    """SIMD issue time of `kernel` from the committed SQ counter summary: vector and matrix instructions take turns
+    on a SIMD of this GPU (2.7 cycles per vector instruction, 32 per v_mfma_f32_16x16x4_f32; measured, see the
+    summary's header), so (2.7 N_vector + 32 N_matrix) / (1024 SIMDs x clock) bounds the kernel from below."""
+    try:
+        for line in open(os.path.join(ROOT, SQ_PROFILE)):
+            f = line.split()
+            if len(f) >= 7 and f[0].split("<")[0] == kernel:
+                mhz, n_valu, n_mfma = float(f[2]), float(f[3]), float(f[6])
+                bound_ms = (2.7 * (n_valu - n_mfma) + 32.0 * n_mfma) / (1024 * mhz * 1e6) * 1e3
+                return {"bound_ms": round(bound_ms, 4), "frac": round(bound_ms / avg_launch_ms, 3), "clock_MHz": mhz,
+                        "vector_instructions": n_valu - n_mfma, "matrix_instructions": n_mfma,
+                        "source": SQ_PROFILE + " (counters of an earlier run, not of this one)"}
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def host_cpu():
     """(model name, physical cores, logical cpus) of the host, from /proc/cpuinfo."""
     model, cores, logical = "unknown", set(), 0
@@ -248,7 +269,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic.get(dominant),
                      "traffic_source": traffic_source,
-                     "algorithmic_bytes_per_launch": algo[dominant], "avg_launch_ms": d_avg_s * 1e3},
+                     "algorithmic_bytes_per_launch": algo[dominant], "avg_launch_ms": d_avg_s * 1e3,
+                     "simd_issue": profiled_issue(dominant, d_avg_s * 1e3)},
         "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
                        "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "kernels": kernels,
