@@ -1221,79 +1221,81 @@ constexpr int kHybMaxTiles = 3;     // 16-column tiles of the m2 axis: degrees u
 // loads, so a unit is better off with one vector wave fewer than the instruction counts suggest.
 constexpr double kHybSlot1Scale = 0.6;
 
-// NK = reduction steps of four rows, NT = 16-column tiles of the m2 axis (1 or 2).  The loop body has
-// no branch: a tile the window of valid m2 does not reach gets zero coefficients.  (With branches
-// around the tiles the compiler copied the accumulators at every join, and each copy waits for
-// the matrix pipeline to drain.)  All addresses are explicit LDS byte addresses advanced by
-// constants from one m to the next.  The table holds zeros where m - m2 is no valid m1 (every
-// table this library fills does), so only the columns past the end of the m2 axis are masked;
-// the fragment column of such an entry is clamped into its row and multiplied by that zero.
-template <int NK, int NT, bool KFULL>
+// x mod n for 0 <= x < 2^20, n < 2^10 (wave-uniform; inv = 1 / n)
+__device__ __forceinline__ int small_mod(int x, int n, float inv) {
+    int r = x - (int)(((float)x + 0.5f) * inv) * n;
+    if (r < 0) r += n;
+    if (r >= n) r -= n;
+    return r;
+}
+
+// NK = reduction steps of four rows; KFULL: the rows fill every step.  One loop per 16-column tile of the m2 axis,
+// over the m indices (of those congruent to `part` modulo `split`) at which one of the tile's columns has a valid
+// m1 = m - m2: a tile outside the window of an m costs nothing, and no branch joins paths that hold the accumulators
+// in different registers (there the compiler copied them, and every copy waits for the matrix pipeline to drain).
+// All addresses are explicit LDS byte addresses advanced by constants from one m to the next.  The table holds zeros
+// where m - m2 is no valid m1 (every table this library fills does), so only the columns past the end of the m2
+// axis are masked; the fragment column of such an entry is clamped into its row and multiplied by that zero.
+template <int NK, bool KFULL>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
-                                            int split, int lane, f32x4 (&dre)[kHybMaxTiles], f32x4 (&dim)[kHybMaxTiles]) {
+                                            int split, float inv_split, int lane, f32x4 (&dre)[kHybMaxTiles],
+                                            f32x4 (&dim)[kHybMaxTiles]) {
     const int l = q.l, l1 = q.l1, l2 = q.l2;
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = q.rows, tau2 = q.tau2;
     const int i = lane & 15, kk = lane >> 4;
     const int io = min(i, tau2 - 1);                              // rows past the last channel repeat it (never stored)
-    // per reduction step: LDS address of the lane's tile entry at m index `part`, base of its fragment row;
-    // rows past the end of the unit repeat the last one and get a zero coefficient
-    unsigned ga[NK], fbase[NK];
+    const int d = l1 + l2 - l;
+    // per reduction step: LDS address of the lane's tile entry at m index 0, base of its fragment row; rows past
+    // the end of the unit repeat the last one and get a zero coefficient
+    unsigned gbase[NK], fbase[NK];
     float kmask[NK];
 #pragma unroll
     for (int c = 0; c < NK; ++c) {
         const int k = 4 * c + kk;
         const int kc = min(k, rows - 1);
         kmask[c] = k < rows ? 1.f : 0.f;
-        ga[c] = opaque(lds_addr(g + (kc * tau2 + io) * M + part));
+        gbase[c] = lds_addr(g + (kc * tau2 + io) * M);
         fbase[c] = lds_addr(f1 + kc * (M1 + 1));
     }
-    // per tile: address of the lane's coefficient at m index `part`, whether its column exists, and
-    // fragment column minus m index (column of slot 1 = m - m2 + l1)
-    unsigned ca[NT];
-    bool colok[NT];
-    int fc0[NT];
+    const int nt = (M2 + 15) >> 4;
+    const unsigned gstep = 8u * (unsigned)split, cstep = 4u * (unsigned)(split * M2);
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
+    for (int t = 0; t < kHybMaxTiles; ++t) {
         const int col = 16 * t + i;
         const int colc = min(col, M2 - 1);
-        colok[t] = col < M2;
-        ca[t] = opaque(lds_addr(cgp + (kTabLo + part) * M2 + colc));
-        fc0[t] = part - l - (colc - l2) + l1;
-    }
-    const unsigned gstep = 8u * (unsigned)split, cstep = 4u * (unsigned)(split * M2);
-    for (int mi = part; mi < M; mi += split) {
-        float2 gq[NK];
-        float ngy[NK];
+        const bool colok = col < M2;
+        // column c of the m2 axis is valid at m index mi iff mi - l - (c - l2) lies in [-l1, l1]
+        const int lo = max(0, 16 * t - d);
+        const int hi = t < nt ? min(M - 1, 16 * t + 15 - d + 2 * l1) : -1;
+        const int mi0 = lo + small_mod(part - lo + 1024 * split, split, inv_split);
+        unsigned ga[NK];
 #pragma unroll
-        for (int c = 0; c < NK; ++c) {
-            gq[c] = lds_c(ga[c], 0);
-            ga[c] += gstep;
-        }
-        float cc[NT];
-        float2 fq[NT][NK];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            cc[t] = lds_f(ca[t])[0];
-            ca[t] += cstep;
-            const int fcol = max(0, min(M1 - 1, fc0[t]));         // clamped where the coefficient is zero anyway
-            fc0[t] += split;
-#pragma unroll
-            for (int c = 0; c < NK; ++c) fq[t][c] = lds_c(fbase[c] + 8u * (unsigned)fcol, 0);
-        }
-#pragma unroll
-        for (int c = 0; c < NK; ++c) ngy[c] = -gq[c].y;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const float cv = (t + 1 < NT) || colok[t] ? cc[t] : 0.f;   // every tile before the last one is full
+        for (int c = 0; c < NK; ++c) ga[c] = opaque(gbase[c] + 8u * (unsigned)mi0);
+        unsigned ca = opaque(lds_addr(cgp + (kTabLo + mi0) * M2 + colc));
+        int fc = mi0 - l - (colc - l2) + l1;                      // fragment column of slot 1 = m - m2 + l1
+        for (int mi = mi0; mi <= hi; mi += split) {
+            float2 gq[NK], fq[NK];
+            const float cc = lds_f(ca)[0];
+            ca += cstep;
+            const int fcol = max(0, min(M1 - 1, fc));             // clamped where the coefficient is zero anyway
+            fc += split;
 #pragma unroll
             for (int c = 0; c < NK; ++c) {
-                const float w = KFULL ? cv : cv * kmask[c];   // KFULL: the rows fill every step of four
-                const float bx = w * fq[t][c].x, by = -w * fq[t][c].y;  // C conj(f)
+                gq[c] = lds_c(ga[c], 0);
+                ga[c] += gstep;
+                fq[c] = lds_c(fbase[c] + 8u * (unsigned)fcol, 0);
+            }
+            const float cv = colok ? cc : 0.f;
+#pragma unroll
+            for (int c = 0; c < NK; ++c) {
+                const float w = KFULL ? cv : cv * kmask[c];
+                const float bx = w * fq[c].x, by = -w * fq[c].y;  // C conj(f)
+                const float ngy = -gq[c].y;
                 dre[t] = mfma4(gq[c].x, bx, dre[t]);
                 dim[t] = mfma4(gq[c].x, by, dim[t]);
-                dre[t] = mfma4(ngy[c], by, dre[t]);
+                dre[t] = mfma4(ngy, by, dre[t]);
                 dim[t] = mfma4(gq[c].y, bx, dim[t]);
             }
         }
@@ -1317,11 +1319,13 @@ __device__ __forceinline__ void bwd_mm_store(const f32x4 (&dre)[kHybMaxTiles], c
     }
 }
 
+template <int NK, bool KFULL>
 __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit& u, BwdUTask t, int part, int split,
                                                   int lane, float2* __restrict__ part2_b) {
     f32x4 dre[kHybMaxTiles], dim[kHybMaxTiles];
 #pragma unroll
     for (int k = 0; k < kHybMaxTiles; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const float inv_split = 1.0f / (float)split;
     int par = 0, f2par = 0;
     for (int ti = u.task_begin; ti < u.task_end; ++ti) {
         BwdUTask cur;
@@ -1329,23 +1333,7 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         const float2 *g, *f2;
         bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
-#define CGNET_MM_CALL(NK_, NT_, KF_) bwd_mm_task<NK_, NT_, KF_>(q, cgp, g, c.f1, part, split, lane, dre, dim)
-#define CGNET_MM_NT(NK_, NT_)                                           \
-    if (u.rows & 3) CGNET_MM_CALL(NK_, NT_, false);                     \
-    else CGNET_MM_CALL(NK_, NT_, true);
-#define CGNET_MM(NK_)                                                   \
-    if (cur.l2 <= 7) { CGNET_MM_NT(NK_, 1) }                            \
-    else if (cur.l2 <= 15) { CGNET_MM_NT(NK_, 2) }                      \
-    else { CGNET_MM_NT(NK_, 3) }
-        switch ((u.rows + 3) >> 2) {
-            case 1: CGNET_MM(1) break;
-            case 2: CGNET_MM(2) break;
-            case 3: CGNET_MM(3) break;
-            default: CGNET_MM(4) break;
-        }
-#undef CGNET_MM_NT
-#undef CGNET_MM_CALL
-#undef CGNET_MM
+        bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, lane, dre, dim);
         if (cur.last_of_l2) {
             const int M2 = 2 * cur.l2 + 1;
             mfma_drain();
@@ -1355,6 +1343,19 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         }
     }
 }
+
+// the matrix-core role for a unit of `rows` rows: reduction steps and whether the rows fill them are fixed per unit
+#define CGNET_HYB_ROLE_B(ROWS_, CALL)                                    \
+    switch ((((ROWS_) + 3) >> 2) * 2 + (((ROWS_) & 3) ? 0 : 1)) {        \
+        case 2: { CALL(1, false); } break;                               \
+        case 3: { CALL(1, true); } break;                                \
+        case 4: { CALL(2, false); } break;                               \
+        case 5: { CALL(2, true); } break;                                \
+        case 6: { CALL(3, false); } break;                               \
+        case 7: { CALL(3, true); } break;                                \
+        case 8: { CALL(4, false); } break;                               \
+        default: { CALL(4, true); } break;                               \
+    }
 
 __global__ void __launch_bounds__(kHybThreads, 4)
 cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
@@ -1397,7 +1398,10 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
         CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
-        bwd_hybrid_loop_b(c, u, t0, wave - u.nA, kHybWaves - u.nA, tid & 63, part2 + (size_t)b * P2);
+#define CGNET_LOOP_B(NK_, KF_) \
+    bwd_hybrid_loop_b<NK_, KF_>(c, u, t0, wave - u.nA, kHybWaves - u.nA, tid & 63, part2 + (size_t)b * P2)
+        CGNET_HYB_ROLE_B(u.rows, CGNET_LOOP_B)
+#undef CGNET_LOOP_B
     }
 }
 
@@ -1581,32 +1585,18 @@ __device__ __forceinline__ void fused_loop_a(const FusedCtx& c, const BwdUnit& u
 }
 
 // Matrix-core waves (slot 2), as bwd_hybrid_loop_b.
+template <int NK, bool KFULL>
 __device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u, const FusedTask* __restrict__ ft,
                                              int part, int split, float2* __restrict__ part2_b) {
     f32x4 dre[kHybMaxTiles], dim[kHybMaxTiles];
 #pragma unroll
     for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const float inv_split = 1.0f / (float)split;
     fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
         const int l2 = ft_l2(t), tau2 = ft_tau2(t);
         const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2};
         const float2* g = reinterpret_cast<const float2*>(c.tile);
-#define CGNET_MM_CALL(NK_, NT_, KF_) bwd_mm_task<NK_, NT_, KF_>(q, cgp, g, c.f1, part, split, c.lane, dre, dim)
-#define CGNET_MM_NT(NK_, NT_)                                           \
-    if (u.rows & 3) CGNET_MM_CALL(NK_, NT_, false);                     \
-    else CGNET_MM_CALL(NK_, NT_, true);
-#define CGNET_MM(NK_)                                                   \
-    if (l2 <= 7) { CGNET_MM_NT(NK_, 1) }                                \
-    else if (l2 <= 15) { CGNET_MM_NT(NK_, 2) }                          \
-    else { CGNET_MM_NT(NK_, 3) }
-        switch ((u.rows + 3) >> 2) {
-            case 1: CGNET_MM(1) break;
-            case 2: CGNET_MM(2) break;
-            case 3: CGNET_MM(3) break;
-            default: CGNET_MM(4) break;
-        }
-#undef CGNET_MM_NT
-#undef CGNET_MM_CALL
-#undef CGNET_MM
+        bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, c.lane, dre, dim);
         if (ft_last(t)) {
             const int M2 = 2 * l2 + 1;
             mfma_drain();
@@ -1668,7 +1658,9 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
         CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
-        fused_loop_b(c, u, ft, wave - u.nA, kHybWaves - u.nA, part2 + (size_t)b * P2);
+#define CGNET_LOOP_B(NK_, KF_) fused_loop_b<NK_, KF_>(c, u, ft, wave - u.nA, kHybWaves - u.nA, part2 + (size_t)b * P2)
+        CGNET_HYB_ROLE_B(u.rows, CGNET_LOOP_B)
+#undef CGNET_LOOP_B
     }
 }
 
