@@ -332,6 +332,7 @@ class CG_woFilter_cuda(nn.Module):
 # --------------------------------------------------------------------------- the whole layer
 _OVERLAP_GRAD_W = int(os.environ.get("CGNET_OVERLAP_GW", "1"))
 _FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "0")))
+_GW_JOIN = os.environ.get("CGNET_GW_JOIN", "auto")     # "early" / "late": where the backward waits for the side stream
 _CU_LDS_BYTES = 160 * 1024
 _side_streams = {}
 
@@ -410,7 +411,10 @@ class _CGBN_fused(torch.autograd.Function):
                 ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
             ctx.wmm_plan.backward(grad_output, grad_FF, None, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
             grad_F = torch.empty_like(Fs)
-            if 2 * ctx.cg_plan.backward_lds + ctx.wmm_plan.gradw_lds > _CU_LDS_BYTES:
+            early = ctx.cg_plan.backward_groups * ctx.cg_plan.backward_lds + ctx.wmm_plan.gradw_lds > _CU_LDS_BYTES
+            if _GW_JOIN != "auto":
+                early = _GW_JOIN == "early"
+            if early:
                 main.wait_stream(side)
             ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
             main.wait_stream(side)

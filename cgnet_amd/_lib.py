@@ -48,6 +48,8 @@ SIGNATURES = {
     "cgnet_CGBN_backward_fused": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                                  ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
+    "cgnet_cg_plan_forward_lds": (ctypes.c_size_t, [_vp]),
+    "cgnet_cg_plan_backward_groups": (ctypes.c_int, [_vp]),
     "cgnet_wmm_plan_gradw_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_profile_enable": (ctypes.c_int, [ctypes.c_int]),
     "cgnet_profile_select": (ctypes.c_int, [ctypes.c_char_p]),

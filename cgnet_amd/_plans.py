@@ -81,6 +81,8 @@ class CGPlan:
         self.t_FF = [int(v) for v in tff]
         self.t_offsets = [int(v) for v in toffs][:len(self.llls)]
         self.backward_lds = int(lib.cgnet_cg_plan_backward_lds(self._h))   # bytes per work-group of the backward
+        self.forward_lds = int(lib.cgnet_cg_plan_forward_lds(self._h))     # ... of the forward (largest launch class)
+        self.backward_groups = int(lib.cgnet_cg_plan_backward_groups(self._h))   # backward work-groups per compute unit
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

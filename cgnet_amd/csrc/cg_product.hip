@@ -149,6 +149,7 @@ constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kBwdPieces = 40;                   // unit backward: a unit holds at most this fraction of a sample's work
 constexpr size_t kMaxHybLds = 80 * 1024;        // hybrid unit backward: two groups of eight waves per CU
+constexpr size_t kHybLds3 = 53 * 1024;          // ... three groups per CU (what its register budget allows)
 constexpr long long kHybTileBytes = 28 * 1024;
 constexpr size_t kMaxUnitLds = 64 * 1024;       // unit backward: LDS-direct copies address the first 64 KB
 
@@ -1043,6 +1044,37 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         }                                                                        \
     }
 
+// slot-1 tilings of the hybrid kernel: at most three output rows per thread (80 registers)
+#define CGNET_BWD_SWITCH_A3(TI_, RW_, RM_, CALL)                                 \
+    if ((RM_) == 2) {                                                            \
+        switch ((TI_) * 32 + (RW_)) {                                            \
+            case 2 * 32 + 4: { CALL(2, 4, 2); } break;                           \
+            case 2 * 32 + 8: { CALL(2, 8, 2); } break;                           \
+            case 2 * 32 + 16: { CALL(2, 16, 2); } break;                         \
+            case 3 * 32 + 4: { CALL(3, 4, 2); } break;                           \
+            case 3 * 32 + 8: { CALL(3, 8, 2); } break;                           \
+            default: { CALL(3, 16, 2); } break;                                  \
+        }                                                                        \
+    } else {                                                                     \
+        switch ((TI_) * 32 + (RW_)) {                                            \
+            case 1 * 32 + 1: { CALL(1, 1, 1); } break;                           \
+            case 1 * 32 + 2: { CALL(1, 2, 1); } break;                           \
+            case 1 * 32 + 4: { CALL(1, 4, 1); } break;                           \
+            case 1 * 32 + 8: { CALL(1, 8, 1); } break;                           \
+            case 1 * 32 + 16: { CALL(1, 16, 1); } break;                         \
+            case 2 * 32 + 1: { CALL(2, 1, 1); } break;                           \
+            case 2 * 32 + 2: { CALL(2, 2, 1); } break;                           \
+            case 2 * 32 + 4: { CALL(2, 4, 1); } break;                           \
+            case 2 * 32 + 8: { CALL(2, 8, 1); } break;                           \
+            case 2 * 32 + 16: { CALL(2, 16, 1); } break;                         \
+            case 3 * 32 + 1: { CALL(3, 1, 1); } break;                           \
+            case 3 * 32 + 2: { CALL(3, 2, 1); } break;                           \
+            case 3 * 32 + 4: { CALL(3, 4, 1); } break;                           \
+            case 3 * 32 + 8: { CALL(3, 8, 1); } break;                           \
+            default: { CALL(3, 16, 1); } break;                                  \
+        }                                                                        \
+    }
+
 struct BwdCtx {
     const float2* Fp;          // this sample's fragments, rows padded with one zero
     const float2* Gb;          // this sample's gFF
@@ -1051,20 +1083,26 @@ struct BwdCtx {
     float2* f1;                // LDS: rows x (M1+1) slab of degree l1 (fixed for the unit)
     char* f2;                  // LDS: two slabs of degree l2 (current run / next run), f2cap bytes each
     char* cg;                  // LDS: two tables, cgcap bytes each
-    char* tile;                // LDS: two tiles, tcap + 16 bytes each
+    char* tile;                // LDS: the tile buffers (two, or one in the hybrid kernel), tcap + 16 bytes each
     int f2cap, cgcap, tcap;
     int tid, rtid;
 };
 
-// Starts the copies of task t: tile and table into buffer `par`, the l2 slab (first task of a
-// run only) into slab buffer `f2par`.
+// Starts the copy of task t's tile into tile buffer `buf`.
 template <int NT>
-__device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, const BwdUTask& t, int par, int f2par) {
-    const int M = 2 * t.l + 1, M2 = 2 * t.l2 + 1;
-    const int ntile = u.rows * t.tau2 * M;
-    char* tile = c.tile + par * (c.tcap + 16);
+__device__ __forceinline__ void bwd_issue_tile(const BwdCtx& c, const BwdUnit& u, const BwdUTask& t, int buf) {
+    const int ntile = u.rows * t.tau2 * (2 * t.l + 1);
+    char* tile = c.tile + buf * (c.tcap + 16);
     dma16<NT>(c.Gb + t.offFF, tile, ntile >> 1, c.tid);
     if (ntile & 1) dma8(c.Gb + t.offFF + (ntile - 1), tile + 8 * (size_t)(ntile - 1), c.tid);
+}
+
+// Starts the copies of task t: table into buffer `par`, the l2 slab (first task of a run only) into slab buffer
+// `f2par`, and with two tile buffers (TWO) the tile into buffer `par`.
+template <int NT, bool TWO>
+__device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, const BwdUTask& t, int par, int f2par) {
+    const int M2 = 2 * t.l2 + 1;
+    if (TWO) bwd_issue_tile<NT>(c, u, t, par);
     dma16<NT>(c.CGP + t.cgp_off, c.cg + par * c.cgcap, t.cgp_len >> 2, c.tid);
     if (t.first_of_l2) dma16<NT>(c.Fp + t.offF2p, c.f2 + f2par * c.f2cap, (t.tau2 * (M2 + 1)) >> 1, c.tid);
 }
@@ -1072,7 +1110,9 @@ __device__ __forceinline__ void bwd_issue(const BwdCtx& c, const BwdUnit& u, con
 // Per-task prologue of both roles.  On entry `t` is the task whose copies were started one
 // task earlier into buffer `par`; on exit they are visible, `cur` holds that task and the
 // copies of the following task are in flight.  One barrier per task, executed by every thread.
-template <int NT>
+// With one tile buffer (TWO = false) the following task's tile is not among those copies: bwd_stage_end starts it
+// when every wave has finished with the current tile (a second barrier per task).
+template <int NT, bool TWO>
 __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int ti, BwdUTask& t, BwdUTask& cur,
                                           int& par, int& f2par, const float*& cgp, const float2*& g,
                                           const float2*& f2) {
@@ -1080,18 +1120,26 @@ __device__ __forceinline__ void bwd_stage(const BwdCtx& c, const BwdUnit& u, int
     __syncthreads();           // copies of every wave landed; nobody still reads the other buffers
     cur = t;
     cgp = reinterpret_cast<const float*>(c.cg + par * c.cgcap);
-    g = reinterpret_cast<const float2*>(c.tile + par * (c.tcap + 16));
+    g = reinterpret_cast<const float2*>(c.tile + (TWO ? par : 0) * (c.tcap + 16));
     f2 = reinterpret_cast<const float2*>(c.f2 + f2par * c.f2cap);
     par ^= 1;
     if (ti + 1 < u.task_end) {
         t = c.tasks[ti + 1];
         if (t.first_of_l2) f2par ^= 1;
-        bwd_issue<NT>(c, u, t, par, f2par);
+        bwd_issue<NT, TWO>(c, u, t, par, f2par);
     }
 }
 
+// Per-task epilogue of both roles with one tile buffer; `t` is the following task (as bwd_stage left it).
+template <int NT, bool TWO>
+__device__ __forceinline__ void bwd_stage_end(const BwdCtx& c, const BwdUnit& u, int ti, const BwdUTask& t) {
+    if (TWO) return;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // every wave's reads of the tile are complete
+    if (ti + 1 < u.task_end) bwd_issue_tile<NT>(c, u, t, 0);
+}
+
 // Waves of role A: gradient of slot 1 (rows of degree l1), kept in registers for the whole unit.
-template <int NT, int TI, int RW, int RM>
+template <int NT, bool TWO, int TI, int RW, int RM>
 __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& u, BwdUTask t,
                                                 float2* __restrict__ dst) {
     float ax[kBwdMaxTI][2], ay[kBwdMaxTI][2], tx[kBwdMaxTI][2], ty[kBwdMaxTI][2];
@@ -1105,9 +1153,10 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         BwdUTask cur;
         const float* cgp;
         const float2 *g, *f2;
-        bwd_stage<NT>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        bwd_stage<NT, TWO>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
         bwd_accum<1, TI, RW, RM>(q, cgp, g, f2, c.rtid, ax, ay);
+        bwd_stage_end<NT, TWO>(c, u, ti, t);
         if (cur.last_of_l2) {
             // blocked summation: the running sum of one l2 is folded into the unit's total
 #pragma unroll
@@ -1134,7 +1183,7 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
         BwdUTask cur;
         const float* cgp;
         const float2 *g, *f2;
-        bwd_stage<kThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        bwd_stage<kThreads, true>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
 #define CGNET_CALL_B(TI_, RW_) bwd_accum<2, TI_, RW_>(q, cgp, g, c.f1, c.rtid, ax, ay)
         CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_CALL_B)
@@ -1151,8 +1200,8 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
 // LDS map (bytes): [16 zero] f1 (f1cap) | f2 x2 (f2cap each) | table x2 (cgcap each) | [16 zero]
 // tile 0 (tcap) [16 zero] tile 1 (tcap) [16 zero].  Everything is cleared once, so positions a
 // tile read may touch just outside the tile hold finite values.
-__host__ __device__ inline size_t bwd_unit_lds(int f1cap, int f2cap, int cgcap, int tcap) {
-    return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + 16 + 2 * ((size_t)tcap + 16);
+__host__ __device__ inline size_t bwd_unit_lds(int f1cap, int f2cap, int cgcap, int tcap, int ntiles = 2) {
+    return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + 16 + ntiles * ((size_t)tcap + 16);
 }
 
 __global__ void __launch_bounds__(kThreads, 4)
@@ -1188,12 +1237,12 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
     __syncthreads();                                 // the clearing stores precede every copy
     const BwdUTask t0 = tasks[u.task_begin];
     dma16<kThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
-    bwd_issue<kThreads>(c, u, t0, 0, 0);
+    bwd_issue<kThreads, true>(c, u, t0, 0, 0);
 
     // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
-#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kThreads, TI_, RW_, RM_>(c, u, t0, dst)
+#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kThreads, true, TI_, RW_, RM_>(c, u, t0, dst)
         CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
@@ -1215,6 +1264,7 @@ constexpr int kHybThreads = 512;
 constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
                                     // slot-2 gradient) slot 2 on the matrix cores
 constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
+constexpr int kHybMaxTI = 3;        // slot 1: output rows per thread (the register budget of three groups per CU)
 constexpr int kHybMaxTiles = 3;     // 16-column tiles of the m2 axis: degrees up to 23
 // Plan: weight of a vector-ALU step of slot 1 against the matrix-core cost of slot 2 in the same
 // work-group.  Measured, not derived: below one because the matrix waves also wait on their operand
@@ -1331,9 +1381,10 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         BwdUTask cur;
         const float* cgp;
         const float2 *g, *f2;
-        bwd_stage<kHybThreads>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
+        bwd_stage<kHybThreads, false>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
         const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
         bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, lane, dre, dim);
+        bwd_stage_end<kHybThreads, false>(c, u, ti, t);
         if (cur.last_of_l2) {
             const int M2 = 2 * cur.l2 + 1;
             mfma_drain();
@@ -1357,7 +1408,7 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         default: { CALL(4, true); } break;                               \
     }
 
-__global__ void __launch_bounds__(kHybThreads, 4)
+__global__ void __launch_bounds__(kHybThreads, 6)     // 80 registers: three work-groups per compute unit
 cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
                           const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                           const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
@@ -1383,19 +1434,20 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
     c.tid = tid;
     c.rtid = tid;                                    // role A: threads 0 .. 64 * nA - 1
     {
-        const int n16 = (int)(bwd_unit_lds(f1cap, f2cap, cgcap, tcap) >> 4);
+        const int n16 = (int)(bwd_unit_lds(f1cap, f2cap, cgcap, tcap, 1) >> 4);
         float4* z = reinterpret_cast<float4*>(smem);
         for (int e = tid; e < n16; e += kHybThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     __syncthreads();                                 // the clearing stores precede every copy
     const BwdUTask t0 = tasks[u.task_begin];
     dma16<kHybThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
-    bwd_issue<kHybThreads>(c, u, t0, 0, 0);
+    bwd_issue<kHybThreads, false>(c, u, t0, 0, 0);
+    bwd_issue_tile<kHybThreads>(c, u, t0, 0);
     // The two roles run the same sequence of barriers (one per task) from different code paths.
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
-#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kHybThreads, TI_, RW_, RM_>(c, u, t0, dst)
-        CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
+#define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kHybThreads, false, TI_, RW_, RM_>(c, u, t0, dst)
+        CGNET_BWD_SWITCH_A3(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
 #define CGNET_LOOP_B(NK_, KF_) \
@@ -1655,7 +1707,7 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
 #define CGNET_LOOP_A(TI_, RW_, RM_) fused_loop_a<TI_, RW_, RM_>(c, u, ft, dst)
-        CGNET_BWD_SWITCH_A(u.TI, u.RW, u.RM, CGNET_LOOP_A)
+        CGNET_BWD_SWITCH_A3(u.TI, u.RW, u.RM, CGNET_LOOP_A)
 #undef CGNET_LOOP_A
     } else {
 #define CGNET_LOOP_B(NK_, KF_) fused_loop_b<NK_, KF_>(c, u, ft, wave - u.nA, kHybWaves - u.nA, part2 + (size_t)b * P2)
@@ -2089,8 +2141,11 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
 
     // ---- register-resident backward: units = (l1, range of t1 rows), tasks ordered by (l2, l)
     std::vector<int> combine_meta, pad_meta;
-    // first with slot 2 on the matrix cores where the shapes allow it, then all on the vector ALUs
-    for (int attempt = 0; attempt < 2 && !p->bwd_fast; ++attempt) {
+    // First with slot 2 on the matrix cores where the shapes allow it: with the largest tiles that still let three
+    // work-groups share a compute unit's LDS (kHybLds3), failing that with two work-groups; then all on the vector ALUs.
+    const int hyb_tiles_kb[] = {40, 36, 32, 28, 24, 20, 16, 12, 8};
+    const int n_hyb = (int)(sizeof(hyb_tiles_kb) / sizeof(hyb_tiles_kb[0]));
+    for (int attempt = 0; attempt < n_hyb + 2 && !p->bwd_fast; ++attempt) {
         bool ok = true;
         int P2 = 0;
         size_t lds_max = 0;
@@ -2104,14 +2159,16 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         }
         // Slot 2 on the matrix cores: needs every channel count to fit one 16-row tile (and to fill a
         // good part of it), the m2 axis kHybMaxTiles 16-column tiles.  CGNET_BWD_HYBRID=0 keeps all on the vector ALUs.
-        bool hybrid = attempt == 0 && n1 - 1 <= 8 * kHybMaxTiles - 1;
+        bool hybrid = attempt <= n_hyb && n1 - 1 <= 8 * kHybMaxTiles - 1;
         for (int l = 0; l < n1; ++l)
             if (h_t_F[l] != 0 && (h_t_F[l] < 8 || h_t_F[l] > 16)) hybrid = false;
         if (const char* e = getenv("CGNET_BWD_HYBRID"); e && e[0] == '0') hybrid = false;
         bool use_rm = true;      // CGNET_BWD_MSPLIT=0: lanes of an item split only the reduced channels
         if (const char* e = getenv("CGNET_BWD_MSPLIT"); e && e[0] == '0') use_rm = false;
-        if (attempt == 0 && !hybrid) continue;
-        const long long tile_limit = hybrid ? kHybTileBytes : kBwdTileBytes;
+        if (attempt <= n_hyb && !hybrid) continue;
+        // attempts 0 .. n_hyb - 1: three groups per compute unit; attempt n_hyb: two groups, tiles of kHybTileBytes
+        const long long tile_limit = !hybrid ? kBwdTileBytes : attempt < n_hyb ? hyb_tiles_kb[attempt] * 1024LL : kHybTileBytes;
+        const size_t hyb_lds_limit = attempt < n_hyb ? kHybLds3 : kMaxHybLds;
         int f1cap = 0, f2cap = 0, cgcap = 0, tcap = 0;
         std::vector<int> own1(n1, 0);
         std::vector<std::vector<int>> lam_offs(n1);
@@ -2169,7 +2226,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     if (!feasible) continue;
                     int max_tau2 = 1;
                     for (int i : tri) max_tau2 = std::max(max_tau2, h_t_F[tl2[i]]);
-                    for (int ti = 1; ti <= kBwdMaxTI; ++ti)
+                    for (int ti = 1; ti <= (hybrid ? kHybMaxTI : kBwdMaxTI); ++ti)
                         for (int rw = 1; rw <= 16; rw *= 2)
                             for (int rm = 1; rm <= 2; ++rm) {
                                 // rm = 2: half of the lanes of an item take the second half of the reduced m range
@@ -2243,7 +2300,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     tcap = std::max(tcap, (int)tile_bytes);
                 }
                 u.task_end = (int)p->bwd_utasks.size();
-                lds_max = bwd_unit_lds(f1cap, f2cap, cgcap, tcap);
+                lds_max = bwd_unit_lds(f1cap, f2cap, cgcap, tcap, hybrid ? 1 : 2);
                 p->bwd_units.push_back(u);
             }
         }
@@ -2295,7 +2352,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         // CGNET_BWD_GENERAL=1 forces the LDS-accumulator kernel (kept for shapes the unit scheme cannot hold)
         const char* force_general = getenv("CGNET_BWD_GENERAL");
         if (force_general && force_general[0] == '1') ok = false;
-        if (ok && !p->bwd_units.empty() && lds_max <= (hybrid ? kMaxHybLds : kMaxUnitLds)) {
+        if (ok && !p->bwd_units.empty() && lds_max <= (hybrid ? hyb_lds_limit : kMaxUnitLds)) {
             p->bwd_hybrid = hybrid;
             // longest units first
             std::vector<int> order(p->bwd_units.size());
@@ -2384,6 +2441,17 @@ extern "C" int cgnet_cg_plan_sizes(const cgnet_cg_plan* plan, int sizes[5]) {
     sizes[3] = plan->cg_len;
     sizes[4] = plan->nllls;
     return CGNET_OK;
+}
+
+extern "C" size_t cgnet_cg_plan_forward_lds(const cgnet_cg_plan* plan) { return plan ? plan->fwd_lds : 0; }
+
+extern "C" int cgnet_cg_plan_backward_groups(const cgnet_cg_plan* plan) {
+    if (!plan) return 0;
+    const size_t lds = cgnet_cg_plan_backward_lds(plan);
+    const int by_lds = lds ? (int)std::min<size_t>(16, cgnet::kMaxLds / lds) : 16;
+    // register budgets: the hybrid kernel 80 registers with eight waves per group, the unit kernel 128 with four
+    const int by_regs = plan->bwd_fast ? (plan->bwd_hybrid ? 3 : 4) : 8;
+    return std::max(1, std::min(by_lds, by_regs));
 }
 
 extern "C" size_t cgnet_cg_plan_backward_lds(const cgnet_cg_plan* plan) {

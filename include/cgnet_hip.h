@@ -82,6 +82,11 @@ int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, int* h_t_offs
  * reference: a scheduling hint for callers that run another kernel on a second stream beside the backward
  * (a compute unit has 160 KB; what two such groups leave decides whether the other kernel fits beside them). */
 size_t cgnet_cg_plan_backward_lds(const cgnet_cg_plan* plan);
+/* The same for the forward kernel (its largest launch class).  No counterpart in the reference. */
+size_t cgnet_cg_plan_forward_lds(const cgnet_cg_plan* plan);
+/* Work-groups of the backward kernel that share a compute unit (its LDS need and register budget decide); with
+ * cgnet_cg_plan_backward_lds the LDS the backward occupies.  No counterpart in the reference. */
+int cgnet_cg_plan_backward_groups(const cgnet_cg_plan* plan);
 
 /* FF = CG product of F with itself over the plan's triples:
  *   FF[b, l, t_off + t1*t_F[l2] + t2, m] = sum_{m1+m2=m} CG * F[b,l1,t1,m1] * F[b,l2,t2,m2].

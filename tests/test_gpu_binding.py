@@ -232,13 +232,15 @@ def test_reference_differential_case(dev):
 
 def test_plans_created_in_descending_lds_order(dev):
     """The dynamic-LDS limit of a kernel belongs to the process, not to the plan created last: a plan whose
-    backward needs more LDS than a later plan's must still launch after that later plan was created."""
+    kernels need more LDS than a later plan's (here the forward's: its work-groups hold whole 16 x 16 x (2l+1)
+    tiles, beyond the 64 KB a kernel gets by default) must still launch after that later plan was created."""
     from cgnet_amd import CG_layers
     shapes = [(20, [16] * 21), (15, [16] * 16), (13, [14] * 14), (11, [12] * 12)]
     mods = [CG_layers.CG_woFilter_cuda(lmax, taus, device=dev) for lmax, taus in shapes]
-    need = [m.native_plan().backward_lds for m in mods]
+    need = [m.native_plan().forward_lds for m in mods]
     assert need[0] > 64 * 1024 and need[0] == max(need), need     # the first plan asks for the most, beyond the default limit
-    assert len(set(need)) > 1, need
+    assert need[-1] < 64 * 1024 and len(set(need)) > 1, need
+    assert len(set(m.native_plan().backward_lds for m in mods)) > 1
     for k in (0, 1, 2, 3, 0):
         lmax, taus = shapes[k]
         x = rand_straight(taus, 1, seed=4).float().to(dev).requires_grad_(True)
