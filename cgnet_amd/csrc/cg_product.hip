@@ -110,6 +110,7 @@ struct cgnet_cg_plan {
     // register-resident backward (used when every unit fits; otherwise the LDS-accumulator kernel)
     bool bwd_fast = false;
     bool bwd_hybrid = false;                     // units run cg_backward_hybrid_kernel (slot 2 on the matrix cores)
+    int bwd_hyb_groups = 0;                      // ... with this many work-groups per compute unit (4, 3 or 2)
     std::vector<cgnet::BwdUnit> bwd_units;
     std::vector<cgnet::BwdUTask> bwd_utasks;
     cgnet::BwdUnit* d_bwd_units = nullptr;
@@ -149,7 +150,8 @@ constexpr int kMaxBwdGroups = 32;
 constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kBwdPieces = 40;                   // unit backward: a unit holds at most this fraction of a sample's work
 constexpr size_t kMaxHybLds = 80 * 1024;        // hybrid unit backward: two groups of eight waves per CU
-constexpr size_t kHybLds3 = 53 * 1024;          // ... three groups per CU (what its register budget allows)
+constexpr size_t kHybLds4 = 39 * 1024;          // ... four groups per CU
+constexpr size_t kHybLds3 = 53 * 1024;          // ... three groups per CU
 constexpr long long kHybTileBytes = 28 * 1024;
 constexpr size_t kMaxUnitLds = 64 * 1024;       // unit backward: LDS-direct copies address the first 64 KB
 
@@ -1044,16 +1046,13 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
         }                                                                        \
     }
 
-// slot-1 tilings of the hybrid kernel: at most three output rows per thread (80 registers)
-#define CGNET_BWD_SWITCH_A3(TI_, RW_, RM_, CALL)                                 \
+// slot-1 tilings of the hybrid kernel: at most two output rows per thread (64 registers)
+#define CGNET_BWD_SWITCH_A2(TI_, RW_, RM_, CALL)                                 \
     if ((RM_) == 2) {                                                            \
         switch ((TI_) * 32 + (RW_)) {                                            \
             case 2 * 32 + 4: { CALL(2, 4, 2); } break;                           \
             case 2 * 32 + 8: { CALL(2, 8, 2); } break;                           \
-            case 2 * 32 + 16: { CALL(2, 16, 2); } break;                         \
-            case 3 * 32 + 4: { CALL(3, 4, 2); } break;                           \
-            case 3 * 32 + 8: { CALL(3, 8, 2); } break;                           \
-            default: { CALL(3, 16, 2); } break;                                  \
+            default: { CALL(2, 16, 2); } break;                                  \
         }                                                                        \
     } else {                                                                     \
         switch ((TI_) * 32 + (RW_)) {                                            \
@@ -1066,13 +1065,30 @@ __device__ __forceinline__ void bwd_flush(int n_o, int M_o, int rtid, float (&ax
             case 2 * 32 + 2: { CALL(2, 2, 1); } break;                           \
             case 2 * 32 + 4: { CALL(2, 4, 1); } break;                           \
             case 2 * 32 + 8: { CALL(2, 8, 1); } break;                           \
-            case 2 * 32 + 16: { CALL(2, 16, 1); } break;                         \
-            case 3 * 32 + 1: { CALL(3, 1, 1); } break;                           \
-            case 3 * 32 + 2: { CALL(3, 2, 1); } break;                           \
-            case 3 * 32 + 4: { CALL(3, 4, 1); } break;                           \
-            case 3 * 32 + 8: { CALL(3, 8, 1); } break;                           \
-            default: { CALL(3, 16, 1); } break;                                  \
+            default: { CALL(2, 16, 1); } break;                                  \
         }                                                                        \
+    }
+
+// ... at most three output rows per thread (80 registers)
+#define CGNET_BWD_SWITCH_A3(TI_, RW_, RM_, CALL)                                 \
+    if ((TI_) == 3) {                                                            \
+        if ((RM_) == 2) {                                                        \
+            switch (RW_) {                                                       \
+                case 4: { CALL(3, 4, 2); } break;                                \
+                case 8: { CALL(3, 8, 2); } break;                                \
+                default: { CALL(3, 16, 2); } break;                              \
+            }                                                                    \
+        } else {                                                                 \
+            switch (RW_) {                                                       \
+                case 1: { CALL(3, 1, 1); } break;                                \
+                case 2: { CALL(3, 2, 1); } break;                                \
+                case 4: { CALL(3, 4, 1); } break;                                \
+                case 8: { CALL(3, 8, 1); } break;                                \
+                default: { CALL(3, 16, 1); } break;                              \
+            }                                                                    \
+        }                                                                        \
+    } else {                                                                     \
+        CGNET_BWD_SWITCH_A2(TI_, RW_, RM_, CALL)                                 \
     }
 
 struct BwdCtx {
@@ -1264,7 +1280,7 @@ constexpr int kHybThreads = 512;
 constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
                                     // slot-2 gradient) slot 2 on the matrix cores
 constexpr int kHybMaxRows = 16;     // reduction steps: at most 4 x 4 rows
-constexpr int kHybMaxTI = 3;        // slot 1: output rows per thread (the register budget of three groups per CU)
+constexpr int kHybMaxTI = 3;        // slot 1: output rows per thread (two where four groups share a compute unit)
 constexpr int kHybMaxTiles = 3;     // 16-column tiles of the m2 axis: degrees up to 23
 // Plan: weight of a vector-ALU step of slot 1 against the matrix-core cost of slot 2 in the same
 // work-group.  Measured, not derived: below one because the matrix waves also wait on their operand
@@ -1408,7 +1424,10 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         default: { CALL(4, true); } break;                               \
     }
 
-__global__ void __launch_bounds__(kHybThreads, 6)     // 80 registers: three work-groups per compute unit
+// G4: 64 registers and at most two output rows per slot-1 thread, so that four work-groups share a compute unit;
+// otherwise 80 registers, three rows, three work-groups (shapes whose tiles would shrink below four rows with four).
+template <bool G4>
+__global__ void __launch_bounds__(kHybThreads, G4 ? 8 : 6)
 cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restrict__ gFF,
                           const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                           const BwdUnit* __restrict__ units, const BwdUTask* __restrict__ tasks,
@@ -1447,7 +1466,11 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
     if (roleA) {
         float2* dst = u.p1off < 0 ? part1 + (size_t)b * nF + u.offF1 : part2 + (size_t)b * P2 + u.p1off;
 #define CGNET_LOOP_A(TI_, RW_, RM_) bwd_unit_loop_a<kHybThreads, false, TI_, RW_, RM_>(c, u, t0, dst)
-        CGNET_BWD_SWITCH_A3(u.TI, u.RW, u.RM, CGNET_LOOP_A)
+        if (G4) {
+            CGNET_BWD_SWITCH_A2(u.TI, u.RW, u.RM, CGNET_LOOP_A)
+        } else {
+            CGNET_BWD_SWITCH_A3(u.TI, u.RW, u.RM, CGNET_LOOP_A)
+        }
 #undef CGNET_LOOP_A
     } else {
 #define CGNET_LOOP_B(NK_, KF_) \
@@ -2141,9 +2164,13 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
 
     // ---- register-resident backward: units = (l1, range of t1 rows), tasks ordered by (l2, l)
     std::vector<int> combine_meta, pad_meta;
-    // First with slot 2 on the matrix cores where the shapes allow it: with the largest tiles that still let three
-    // work-groups share a compute unit's LDS (kHybLds3), failing that with two work-groups; then all on the vector ALUs.
-    const int hyb_tiles_kb[] = {40, 36, 32, 28, 24, 20, 16, 12, 8};
+    // First with slot 2 on the matrix cores where the shapes allow it: with the largest tiles that let four work-groups
+    // share a compute unit's LDS (kHybLds4) unless that cuts a degree's tiles below four rows, then the same for three
+    // groups (kHybLds3), failing that with two work-groups; then all on the vector ALUs.  Measured at tau = 16:
+    // L=15, four groups with 5-row tiles 1.54 ms, three groups with 10-row tiles 1.57 ms; L=20 (B=16), four groups with
+    // 2-row tiles 1.96 ms, three groups with 4-row tiles 1.44 ms.
+    const int hyb_tiles_kb[] = {30, 28, 24, 20, 16, 12, 40, 36, 32, 28, 24, 20, 16, 12, 8, 4};
+    const int n_hyb4 = 6;
     const int n_hyb = (int)(sizeof(hyb_tiles_kb) / sizeof(hyb_tiles_kb[0]));
     for (int attempt = 0; attempt < n_hyb + 2 && !p->bwd_fast; ++attempt) {
         bool ok = true;
@@ -2166,9 +2193,12 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         bool use_rm = true;      // CGNET_BWD_MSPLIT=0: lanes of an item split only the reduced channels
         if (const char* e = getenv("CGNET_BWD_MSPLIT"); e && e[0] == '0') use_rm = false;
         if (attempt <= n_hyb && !hybrid) continue;
-        // attempts 0 .. n_hyb - 1: three groups per compute unit; attempt n_hyb: two groups, tiles of kHybTileBytes
+        // attempts 0 .. n_hyb4 - 1: four groups per compute unit; .. n_hyb - 1: three; attempt n_hyb: two groups, tiles
+        // of kHybTileBytes
+        const int hyb_groups = attempt < n_hyb4 ? 4 : attempt < n_hyb ? 3 : 2;
         const long long tile_limit = !hybrid ? kBwdTileBytes : attempt < n_hyb ? hyb_tiles_kb[attempt] * 1024LL : kHybTileBytes;
-        const size_t hyb_lds_limit = attempt < n_hyb ? kHybLds3 : kMaxHybLds;
+        const size_t hyb_lds_limit = hyb_groups == 4 ? kHybLds4 : hyb_groups == 3 ? kHybLds3 : kMaxHybLds;
+        const int hyb_max_ti = hyb_groups == 4 ? 2 : kHybMaxTI;
         int f1cap = 0, f2cap = 0, cgcap = 0, tcap = 0;
         std::vector<int> own1(n1, 0);
         std::vector<std::vector<int>> lam_offs(n1);
@@ -2226,7 +2256,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                     if (!feasible) continue;
                     int max_tau2 = 1;
                     for (int i : tri) max_tau2 = std::max(max_tau2, h_t_F[tl2[i]]);
-                    for (int ti = 1; ti <= (hybrid ? kHybMaxTI : kBwdMaxTI); ++ti)
+                    for (int ti = 1; ti <= (hybrid ? hyb_max_ti : kBwdMaxTI); ++ti)
                         for (int rw = 1; rw <= 16; rw *= 2)
                             for (int rm = 1; rm <= 2; ++rm) {
                                 // rm = 2: half of the lanes of an item take the second half of the reduced m range
@@ -2257,6 +2287,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 }
             }
             if (best.total < 0) { ok = false; break; }
+            // four groups per compute unit only while every degree keeps tiles of at least four rows
+            if (hybrid && hyb_groups == 4 && best.rows < std::min(tau1, 4)) { ok = false; break; }
             for (int r0 = 0; r0 < tau1; r0 += best.rows) {
                 BwdUnit u;
                 u.l1 = l1;
@@ -2354,6 +2386,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         if (force_general && force_general[0] == '1') ok = false;
         if (ok && !p->bwd_units.empty() && lds_max <= (hybrid ? hyb_lds_limit : kMaxUnitLds)) {
             p->bwd_hybrid = hybrid;
+            p->bwd_hyb_groups = hybrid ? hyb_groups : 0;
             // longest units first
             std::vector<int> order(p->bwd_units.size());
             for (size_t k = 0; k < order.size(); ++k) order[k] = (int)k;
@@ -2415,7 +2448,9 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         CGNET_HIP(hipMemcpy(p->d_bwd_combine, combine_meta.data(), sizeof(int) * combine_meta.size(), hipMemcpyHostToDevice));
         CGNET_HIP(hipMalloc((void**)&p->d_bwd_padmeta, sizeof(int) * pad_meta.size()));
         CGNET_HIP(hipMemcpy(p->d_bwd_padmeta, pad_meta.data(), sizeof(int) * pad_meta.size(), hipMemcpyHostToDevice));
-        if (int rc = raise_dynamic_lds(p->bwd_hybrid ? (const void*)cg_backward_hybrid_kernel : (const void*)cg_backward_unit_kernel,
+        if (int rc = raise_dynamic_lds(!p->bwd_hybrid            ? (const void*)cg_backward_unit_kernel
+                                       : p->bwd_hyb_groups == 4 ? (const void*)cg_backward_hybrid_kernel<true>
+                                                                : (const void*)cg_backward_hybrid_kernel<false>,
                                        p->bwd_fast_lds))
             return rc;
     }
@@ -2449,8 +2484,8 @@ extern "C" int cgnet_cg_plan_backward_groups(const cgnet_cg_plan* plan) {
     if (!plan) return 0;
     const size_t lds = cgnet_cg_plan_backward_lds(plan);
     const int by_lds = lds ? (int)std::min<size_t>(16, cgnet::kMaxLds / lds) : 16;
-    // register budgets: the hybrid kernel 80 registers with eight waves per group, the unit kernel 128 with four
-    const int by_regs = plan->bwd_fast ? (plan->bwd_hybrid ? 3 : 4) : 8;
+    // register budgets: the hybrid kernel 64 or 80 registers with eight waves per group, the unit kernel 128 with four
+    const int by_regs = !plan->bwd_fast ? 8 : plan->bwd_hybrid ? std::max(2, std::min(4, plan->bwd_hyb_groups)) : 4;
     return std::max(1, std::min(by_lds, by_regs));
 }
 
@@ -2623,8 +2658,13 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
         CGNET_HIP(hipGetLastError());
         CGNET_REQUIRE((long long)B * (long long)plan->bwd_units.size() < (1LL << 31), CGNET_ERR_UNSUPPORTED,
                       "%d samples x %zu units exceed the grid limit", B, plan->bwd_units.size());
-        if (plan->bwd_hybrid) {
-            CGNET_LAUNCH(cg_backward_hybrid_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads),
+        if (plan->bwd_hybrid && plan->bwd_hyb_groups == 4) {
+            CGNET_LAUNCH(cg_backward_hybrid_kernel<true>, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads),
+                         plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
+                         plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
+                         plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
+        } else if (plan->bwd_hybrid) {
+            CGNET_LAUNCH(cg_backward_hybrid_kernel<false>, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads),
                          plan->bwd_fast_lds, s, (const float2*)Fp, (const float2*)d_gFF, (const float*)CGP, part1, part2,
                          plan->d_bwd_units, plan->d_bwd_utasks, plan->nF, plan->bwd_nFp, plan->nFF, plan->bwd_P2,
                          plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, B);
