@@ -1496,8 +1496,9 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
 // x 16 real columns (one accumulator each), numbered column-tile major, and every wave takes a contiguous share.
 // Phase 2: the tile is used exactly as in the hybrid kernel (slot 1 on the vector ALUs, slot 2 on the matrix
 // cores).  The two operands of the next task's tile are copied into LDS during phase 2 (their buffers are only read
-// in phase 1), its coefficient table and l2 slab during the whole stage (double-buffered).  A wave learns about the
-// task after the next one through scalar loads that are in flight for a whole stage.
+// in phase 1); the task's own coefficient table and l2 slab, which only phase 2 reads, are copied during its phase 1.
+// Every buffer exists once, which keeps the work-group small enough for three to share a compute unit.  A wave
+// learns about the task after the next one through scalar loads that are in flight for a whole stage.
 __device__ __forceinline__ void lds_barrier() {      // this wave's LDS accesses are complete, then the group's barrier
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -1606,27 +1607,23 @@ template <typename Work>
 __device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTask* __restrict__ ft, int ntask, Work work) {
     FusedTask cur = ft[0];
     FusedTask nxt = ft[min(1, ntask - 1)];
-    int f2par = 0;
     for (int k = 0; k < ntask; ++k) {
         dma_wait();
-        __syncthreads();       // everything copied for this stage has landed; nobody uses the tile or the other buffers
+        __syncthreads();       // the tile's operands have landed; nobody uses the tile, the table or the l2 slab
         const FusedTask nxt2 = ft[min(k + 2, ntask - 1)];        // needed at the next stage
         const bool more = k + 1 < ntask;
-        const int b = k & 1;
-        if (more) {
-            dma16<kHybThreads>(c.CGP + nxt.cgp_off, c.cg + (b ^ 1) * c.cgcap, nxt.cgp_len >> 2, c.tid);
-            if (ft_first(nxt))
-                dma16<kHybThreads>(c.Fp + nxt.offF2p, c.f2 + (f2par ^ 1) * c.f2cap,
-                                   (ft_tau2(nxt) * (2 * ft_l2(nxt) + 2)) >> 1, c.tid);
-        }
+        // this stage's table and (at the start of a run) l2 slab are only read in phase 2: they arrive during phase 1
+        dma16<kHybThreads>(c.CGP + cur.cgp_off, c.cg, cur.cgp_len >> 2, c.tid);
+        if (ft_first(cur) || k == 0)
+            dma16<kHybThreads>(c.Fp + cur.offF2p, c.f2, (ft_tau2(cur) * (2 * ft_l2(cur) + 2)) >> 1, c.tid);
         gen_phase(cur, c.al, c.bl, c.tile, c.wave, c.lane);
-        lds_barrier();         // the tile is complete; the operand buffers are free
+        dma_wait();
+        lds_barrier();         // the tile is complete, table and slab have landed; the operand buffers are free
         if (more) {
             dma16<kHybThreads>(c.Ag + nxt.aoff, c.al, nxt.chunks & 0xffff, c.tid);
             dma16<kHybThreads>(c.Bg + nxt.boff, c.bl, nxt.chunks >> 16, c.tid);
         }
-        work(cur, reinterpret_cast<const float*>(c.cg + b * c.cgcap), reinterpret_cast<const float2*>(c.f2 + f2par * c.f2cap));
-        if (more && ft_first(nxt)) f2par ^= 1;
+        work(cur, reinterpret_cast<const float*>(c.cg), reinterpret_cast<const float2*>(c.f2));
         cur = nxt;
         nxt = nxt2;
     }
@@ -1682,12 +1679,12 @@ __device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u
     });
 }
 
-// LDS map (bytes): [16 zero] f1 | f2 x2 | table x2 | B operand | A operand | [16 zero] tile [16 zero]
+// LDS map (bytes): [16 zero] f1 | f2 | table | B operand | A operand | [16 zero] tile [16 zero]
 __host__ __device__ inline size_t bwd_fused_lds(int f1cap, int f2cap, int cgcap, int tcap, int bcap, int acap) {
-    return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + (size_t)bcap + (size_t)acap + 16 + (size_t)tcap + 16;
+    return 16 + (size_t)f1cap + (size_t)f2cap + (size_t)cgcap + (size_t)bcap + (size_t)acap + 16 + (size_t)tcap + 16;
 }
 
-__global__ void __launch_bounds__(kHybThreads, 4)
+__global__ void __launch_bounds__(kHybThreads, 6)     // 80 registers: three work-groups per compute unit where the LDS allows
 cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restrict__ Bg, const float* __restrict__ Ag,
                            const float* __restrict__ CGP, float2* __restrict__ part1, float2* __restrict__ part2,
                            const BwdUnit* __restrict__ units, const FusedTask* __restrict__ ftasks, int nF, int nFp,
@@ -1707,8 +1704,8 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
     c.CGP = CGP;
     c.f1 = reinterpret_cast<float2*>(smem + 16);
     c.f2 = reinterpret_cast<char*>(smem) + 16 + f1cap;
-    c.cg = c.f2 + 2 * f2cap;
-    c.bl = reinterpret_cast<float*>(c.cg + 2 * cgcap);
+    c.cg = c.f2 + f2cap;
+    c.bl = reinterpret_cast<float*>(c.cg + cgcap);
     c.al = reinterpret_cast<float*>(reinterpret_cast<char*>(c.bl) + bcap);
     c.tile = reinterpret_cast<float*>(reinterpret_cast<char*>(c.al) + acap + 16);
     c.f2cap = f2cap; c.cgcap = cgcap;
@@ -1722,8 +1719,6 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
     const FusedTask* ft = ftasks + u.task_begin;
     const FusedTask t0 = ft[0];
     dma16<kHybThreads>(c.Fp + u.offF1p, c.f1, (u.rows * (M1 + 1)) >> 1, tid);
-    dma16<kHybThreads>(c.CGP + t0.cgp_off, c.cg, t0.cgp_len >> 2, tid);
-    dma16<kHybThreads>(c.Fp + t0.offF2p, c.f2, (ft_tau2(t0) * (2 * ft_l2(t0) + 2)) >> 1, tid);
     dma16<kHybThreads>(c.Ag + t0.aoff, c.al, t0.chunks & 0xffff, tid);
     dma16<kHybThreads>(c.Bg + t0.boff, c.bl, t0.chunks >> 16, tid);
     // the first stage waits for these copies
