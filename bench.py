@@ -145,6 +145,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--fused-backward", action="store_true",
+                    help="run the layer's backward in one kernel, without grad_FF in memory (default: two kernels)")
     ap.add_argument("--cpu-batch", type=int, default=16)
     ap.add_argument("--cpu-repeats", type=int, default=6)
     ap.add_argument("--copy-probe", action="store_true",
@@ -166,6 +168,8 @@ def main():
     lmax, tau, bsz = WORKLOAD["lmax"], WORKLOAD["tau"], WORKLOAD["batch"]
     taus = [tau] * (lmax + 1)
     layer = CG_layers.CGBN_cuda(lmax, taus, taus, batchnorm=True, sparse_flag=False, device=dev)
+    if args.fused_backward:
+        layer.fused_backward = True
     t_ff = [int(v) for v in layer.t_FF]
     x, w, go = synthetic(lmax, tau, bsz, t_ff)
     with torch.no_grad():
@@ -209,8 +213,9 @@ def main():
     survey = _lib.kernel_times()
     # timed region: only the dominant kernel is bracketed (each event pair costs a few microseconds)
     lib.cgnet_profile_reset()
-    candidates = ("cg_forward_kernel", "wmm_forward_kernel", "wmm_gradw_kernel", "wmm_gradff_mfma_kernel",
-                  "wmm_gradff_kernel", "cg_backward_unit_kernel", "cg_backward_hybrid_kernel", "cg_backward_kernel")
+    candidates = ("cg_forward_kernel", "cg_forward_mm_kernel", "wmm_forward_kernel", "wmm_gradw_kernel",
+                  "wmm_gradff_mfma_kernel", "wmm_gradff_kernel", "cg_backward_unit_kernel", "cg_backward_hybrid_kernel",
+                  "cg_backward_kernel", "cgbn_backward_fused_kernel")
     dominant = max((n for n in survey if n in candidates), key=lambda n: survey[n][0])
     lib.cgnet_profile_select(dominant.encode())
     lib.cgnet_profile_enable(1)
@@ -234,6 +239,7 @@ def main():
     # algorithmic bytes per launch of the five kernels that stream the product tensor
     algo = {
         "cg_forward_kernel": 8 * bsz * (n_f + n_ff),
+        "cg_forward_mm_kernel": 8 * bsz * (n_f + n_ff),
         "wmm_forward_kernel": 8 * (bsz * n_ff + n_w + bsz * n_o) + 4 * sum_t,
         "wmm_gradw_kernel": 8 * (bsz * n_ff + bsz * n_o + n_w),
         "wmm_gradff_mfma_kernel": 8 * (bsz * n_o + n_w + bsz * n_ff),
@@ -242,6 +248,9 @@ def main():
         "cg_backward_hybrid_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
+    # the one-kernel layer backward stands for two of the five passes (grad FF written, grad FF read); it is priced
+    # against the bytes those passes would move although it moves neither
+    algo["cgbn_backward_fused_kernel"] = algo["wmm_gradff_mfma_kernel"] + algo["cg_backward_hybrid_kernel"]
     measured_traffic, traffic_source = profiled_traffic()
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
     kernels = {}
@@ -273,6 +282,7 @@ def main():
                      "simd_issue": profiled_issue(dominant, d_avg_s * 1e3)},
         "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
                        "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "fused_backward": bool(layer.fused_backward),
         "kernels": kernels,
         "kernels_note": "per-kernel table from %d untimed steps with every launch bracketed by events; "
                         "in the timed steps only the dominant kernel is bracketed" % survey_steps,
