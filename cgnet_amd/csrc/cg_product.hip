@@ -1214,8 +1214,8 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
 }
 
 // LDS map (bytes): [16 zero] f1 (f1cap) | f2 x2 (f2cap each) | table x2 (cgcap each) | [16 zero]
-// tile 0 (tcap) [16 zero] tile 1 (tcap) [16 zero].  Everything is cleared once, so positions a
-// tile read may touch just outside the tile hold finite values.
+// tile 0 (tcap) [16 zero] tile 1 (tcap) [16 zero]; the hybrid kernel has tile 0 only.  Everything is cleared
+// once, so positions a tile read may touch just outside the tile hold finite values.
 __host__ __device__ inline size_t bwd_unit_lds(int f1cap, int f2cap, int cgcap, int tcap, int ntiles = 2) {
     return 16 + (size_t)f1cap + 2 * (size_t)f2cap + 2 * (size_t)cgcap + 16 + ntiles * ((size_t)tcap + 16);
 }
@@ -1271,11 +1271,13 @@ cg_backward_unit_kernel(const float2* __restrict__ Fp, const float2* __restrict_
 //   gF2[t2, m2] += sum_t1 G_m[t1, t2] * (C[m][m2] conj F1[t1][m - m2])       (tau2 x rows)(rows x window of m2)
 // is a small matrix product: rows of the accumulator = the up to 16 channels of degree l2, columns
 // = up to three tiles of 16 values of m2, reduction over the up to 16 rows of the unit in steps of 4.
-// Work-groups of eight waves: waves 0-3 keep the slot-1 gradient on the vector ALUs exactly as in
-// cg_backward_unit_kernel, waves 4-7 take slot 2 here, each every fourth m.  The two halves use
-// different pipelines of the same SIMDs (a wave of either half on each), so the vector ALUs carry
-// about half the arithmetic.  The four partial slot-2 gradients leave as separate slabs;
-// cg_backward_combine_kernel adds them.
+// Work-groups of eight waves: the first nA keep the slot-1 gradient on the vector ALUs exactly as in
+// cg_backward_unit_kernel, the others take slot 2 here, each every (8 - nA)-th m.  A matrix instruction costs
+// the SIMD fewer issue cycles per useful product than the vector route does (the two kinds take turns on a SIMD,
+// they do not run side by side), so the vector ALUs carry about half the arithmetic.  The partial slot-2 gradients
+// of the matrix waves leave as separate slabs; cg_backward_combine_kernel adds them.  The kernel keeps one tile
+// buffer and few registers, so that three or four work-groups share a compute unit: its waves wait for LDS reads
+// and for each other (two barriers per task), and it is other work-groups that fill those waits.
 constexpr int kHybThreads = 512;
 constexpr int kHybWaves = 8;        // the first BwdUnit::nA of them take slot 1, the others (= partial slabs per
                                     // slot-2 gradient) slot 2 on the matrix cores
