@@ -259,6 +259,23 @@ def test_cg_random_shapes_matrix_core_backward(dev, lmax, taus, bsz, mode):
     test_cg_forward_backward(dev, lmax, taus, bsz, mode)
 
 
+def _random_matrix_core_cases_high(n, seed):
+    """The same at degrees 8..13 with ragged channel counts (row blocks cut by the LDS budget, partial last
+    reduction steps, two column tiles); spanning-tree or two-pair triple lists keep the oracle in seconds."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        lmax = int(rng.integers(8, 14))
+        taus = [int(rng.integers(8, 17)) for _ in range(lmax + 1)]
+        cases.append((lmax, taus, int(rng.integers(1, 4)), str(rng.choice(["mst", "debug"]))))
+    return cases
+
+
+@pytest.mark.parametrize("lmax,taus,bsz,mode", _random_matrix_core_cases_high(6, 9))
+def test_cg_random_shapes_matrix_core_high_degrees(dev, lmax, taus, bsz, mode):
+    test_cg_forward_backward(dev, lmax, taus, bsz, mode)
+
+
 @pytest.mark.parametrize("lmax,taus,bsz,mode", [CG_CASES[2], CG_CASES[5], CG_CASES[7]])
 def test_cg_backward_general_kernel(dev, monkeypatch, lmax, taus, bsz, mode):
     """The LDS-accumulator backward kernel (fallback for shapes the register-resident scheme cannot
