@@ -190,6 +190,30 @@ def precomputeCG(lmax, method='mst', device='cuda'):
     raise NotImplementedError()
 
 
+def _straight(fragments):
+    """List over l of (B, tau[l], 2l+1, 2) GPU tensors -> the straight tensor (B, sum tau[l](2l+1), 2).  When the
+    fragments are the consecutive views ``CGutils.reshape_out`` makes of one straight tensor (what a stack of these
+    layers hands from one to the next), that tensor is returned as it is; otherwise the fragments are concatenated
+    (reference: CGNet/CG_layers.py:275)."""
+    first = fragments[0]
+    assert first.is_cuda
+    B = first.shape[0]
+    base = first._base
+    if base is not None and base.dim() == 3 and base.shape[0] == B and base.shape[2] == 2 and base.is_contiguous():
+        off, ok = base.storage_offset(), True
+        row = base.shape[1] * 2
+        for v in fragments:
+            n = v.numel() // B if B else 0
+            if (v._base is not base or v.dim() != 4 or v.shape[0] != B or v.shape[3] != 2
+                    or v.storage_offset() != off or v.stride() != (row, v.shape[2] * 2, 2, 1)):
+                ok = False
+                break
+            off += n
+        if ok and off - base.storage_offset() == row:
+            return base
+    return torch.cat([v.reshape(B, -1, 2) for v in fragments], dim=1)
+
+
 # --------------------------------------------------------------------------- CG product
 class _CG_sparse_cuda(torch.autograd.Function):
     @staticmethod
@@ -314,9 +338,7 @@ class CG_woFilter_cuda(nn.Module):
         """``activations``: list over l of (B, tau[l], 2l+1, 2) GPU tensors, or the straight
         tensor (B, sum tau[l](2l+1), 2).  Returns the straight product, or its list form."""
         if isinstance(activations, (list, tuple)):
-            B = activations[0].shape[0]
-            assert activations[0].is_cuda
-            new_activations = torch.cat([v.reshape(B, -1, 2) for v in activations], dim=1)
+            new_activations = _straight(activations)
         else:
             new_activations = activations
         assert new_activations.is_cuda
@@ -330,101 +352,59 @@ class CG_woFilter_cuda(nn.Module):
 
 
 # --------------------------------------------------------------------------- the whole layer
-_OVERLAP_GRAD_W = int(os.environ.get("CGNET_OVERLAP_GW", "1"))
-_FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "0")))
-_GW_JOIN = os.environ.get("CGNET_GW_JOIN", "auto")     # "early" / "late": where the backward waits for the side stream
-_CU_LDS_BYTES = 160 * 1024
-_side_streams = {}
-
-
-def _side_stream(device):
-    key = torch.device(device).index
-    if key not in _side_streams:
-        _side_streams[key] = torch.cuda.Stream(device=device)
-    return _side_streams[key]
+# CGNET_FUSED_BACKWARD=0: new layers take the two-kernel backward (grad_FF in memory) even where the one-kernel
+# backward is available
+_FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "1")))
 
 
 class _CGBN_fused(torch.autograd.Function):
-    """CG product -> fragment norm -> weight mixing in one autograd node.  Same arithmetic as
-    ``_CG_sparse_cuda`` followed by ``_MyBatchNormWeightMM_cuda``; the only difference is that the
-    per-channel statistics come out of the product kernel instead of a second pass over FF."""
+    """CG product -> fragment norm -> weight mixing in one autograd node (``cgnet_CGBN_forward``).  Same
+    arithmetic and results as ``_CG_sparse_cuda`` followed by ``_MyBatchNormWeightMM_cuda``; the per-channel
+    statistics come out of the product kernel instead of a second pass over FF, and neither FF nor grad_FF is
+    visible outside the node, so the backward may skip grad_FF altogether (``fused_backward``)."""
 
     @staticmethod
-    def forward(ctx, Fs, W, cg_plan, wmm_plan, CG, bn_stds, bn_cnt, bn_eps, training, fused_backward=False):
-        ctx.fused_backward = bool(fused_backward)
+    def forward(ctx, Fs, W, layer_plan, CG, bn_stds, bn_cnt, bn_eps, training, fused_backward=True):
+        cg_plan, wmm_plan = layer_plan.cg_plan, layer_plan.wmm_plan
         Fs = Fs.contiguous()
         W = W.contiguous()
         B = Fs.shape[0]
         dev = Fs.device
         flags = (BN_FLAG if bn_stds is not None else 0) | (UPDATESTD_FLAG if training else 0)
         FF = torch.empty(B, cg_plan.nFF, 2, device=dev, dtype=torch.float)
-        sums = None
-        if bn_stds is not None and training:
-            sums = torch.empty(cg_plan.sum_tFF, 2, device=dev, dtype=torch.float64)
-            cg_plan.forward_stats(Fs, FF, CG, B, sums)
-        else:
-            cg_plan.forward(Fs, FF, CG, B)
         out = torch.empty(B, wmm_plan.nO, 2, device=dev, dtype=torch.float)
-        wmm_plan.forward(FF, out, W, B, bn_stds, float(bn_cnt), float(bn_eps), flags, sums)
-        saved_stds = bn_stds.detach().clone() if bn_stds is not None else None
-        ctx.cg_plan, ctx.wmm_plan, ctx.B, ctx.eps, ctx.flags = cg_plan, wmm_plan, B, float(bn_eps), flags
-        ctx.save_for_backward(Fs, W, FF, CG, saved_stds)
+        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        ctx.fused_backward = bool(fused_backward) and layer_plan.fused_backward_supported
+        # the operands of the one-kernel backward are prepared beside those of the mixing forward, in the same launch
+        saved_ops = layer_plan.forward(Fs, FF, out, W, CG, B, bn_stds, float(bn_cnt), float(bn_eps), flags,
+                                       save=ctx.fused_backward and ctx.needs_input_grad[0])
+        # bn_stds was updated in place; backward must see the value used for this batch
+        saved_stds = bn_stds.detach().clone() if (bn_stds is not None and need_grad) else None
+        ctx.layer_plan, ctx.B, ctx.eps, ctx.flags = layer_plan, B, float(bn_eps), flags
+        ctx.save_for_backward(Fs, W, FF, CG, saved_stds, saved_ops)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        Fs, W, FF, CG, stds = ctx.saved_tensors
+        Fs, W, FF, CG, stds, saved_ops = ctx.saved_tensors
+        cg_plan, wmm_plan = ctx.layer_plan.cg_plan, ctx.layer_plan.wmm_plan
         grad_output = grad_output.contiguous()
         need_F, need_W = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         grad_W = torch.empty_like(W) if need_W else None
-        grad_F = None
-        if need_F and ctx.fused_backward and _plans.fused_backward_supported(ctx.cg_plan, ctx.wmm_plan):
-            # The gradient with respect to FF never exists in memory: the product's backward forms every
-            # tile of it in LDS from grad_output and the weights.  The weight gradient (which needs FF, not
-            # gFF) runs beside it on the second stream.
-            main = torch.cuda.current_stream(Fs.device)
-            overlap = need_W and _OVERLAP_GRAD_W
+        grad_F = torch.empty_like(Fs) if need_F else None
+        if need_F and ctx.fused_backward:
+            # The gradient with respect to FF never exists in memory: the product's backward forms every tile of
+            # it in LDS from grad_output and the weights.  The weight gradient needs FF, not grad_FF.
             if need_W:
-                side = _side_stream(Fs.device) if overlap else main
-                if overlap:
-                    side.wait_stream(main)
-                with torch.cuda.stream(side):
-                    ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
-            grad_F = torch.empty_like(Fs)
-            _plans.fused_backward(ctx.cg_plan, ctx.wmm_plan, Fs, grad_F, grad_output, W, CG, ctx.B, stds, ctx.eps,
-                                  ctx.flags)
-            if overlap:
-                main.wait_stream(side)
-            return grad_F, grad_W, None, None, None, None, None, None, None, None
+                wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
+            ctx.layer_plan.backward_fused(Fs, grad_F, grad_output, W, CG, ctx.B, stds, ctx.eps, ctx.flags, saved_ops)
+            return grad_F, grad_W, None, None, None, None, None, None, None
         grad_FF = torch.empty_like(FF) if need_F else None
-        if need_F and need_W and _OVERLAP_GRAD_W:
-            # The weight gradient depends on nothing the other chain produces: it runs on a second
-            # stream (default priority) beside grad FF.  Its tail may run into the CG backward only
-            # when one of its work-groups fits into the LDS two groups of that kernel leave on a
-            # compute unit (160 KB); otherwise the two kernels take turns on the compute units and
-            # the CG backward loses more than the overlap gains, so the side stream is joined first.
-            # CGNET_OVERLAP_GW=0 keeps the whole backward on one stream.
-            main = torch.cuda.current_stream(Fs.device)
-            side = _side_stream(Fs.device)
-            side.wait_stream(main)
-            with torch.cuda.stream(side):
-                ctx.wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
-            ctx.wmm_plan.backward(grad_output, grad_FF, None, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
-            grad_F = torch.empty_like(Fs)
-            early = ctx.cg_plan.backward_groups * ctx.cg_plan.backward_lds + ctx.wmm_plan.gradw_lds > _CU_LDS_BYTES
-            if _GW_JOIN != "auto":
-                early = _GW_JOIN == "early"
-            if early:
-                main.wait_stream(side)
-            ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
-            main.wait_stream(side)
-            return grad_F, grad_W, None, None, None, None, None, None, None, None
         if need_F or need_W:
-            ctx.wmm_plan.backward(grad_output, grad_FF, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
+            wmm_plan.backward(grad_output, grad_FF, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
         if need_F:
-            grad_F = torch.empty_like(Fs)
-            ctx.cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
-        return grad_F, grad_W, None, None, None, None, None, None, None, None
+            cg_plan.backward(Fs, grad_F, grad_FF, CG, ctx.B)
+        return grad_F, grad_W, None, None, None, None, None, None, None
 
 
 class CGBN_cuda(nn.Module):
@@ -443,21 +423,28 @@ class CGBN_cuda(nn.Module):
         self.fused = True      # False: chain the two reference Functions (separate statistics pass)
         # With ``fused``: True takes the backward from grad_output to the input gradient in one kernel, without a
         # grad_FF tensor (B x nFF complex) in memory, where the shapes allow it
-        # (cgnet_CGBN_backward_fused_supported); same gradients, bit for bit.  Off by default: at the benchmark
-        # shape it saves the memory but no time yet (CGNET_FUSED_BACKWARD=1 turns it on for new layers).
+        # (cgnet_CGBN_backward_fused_supported); False keeps the two-kernel backward.  Same gradients either way.
         self.fused_backward = _FUSED_BACKWARD
+        self._layer_plan = None
         self.to(device)
+
+    def native_layer_plan(self):
+        """The native layer plan (product plan linked with the mixing plan), created on first use and again
+        whenever one of the two plans has been rebuilt (a move to another device)."""
+        cg_plan, wmm_plan = self.cg.native_plan(), self.bnWMM.native_plan()
+        lp = self._layer_plan
+        if lp is None or lp.cg_plan is not cg_plan or lp.wmm_plan is not wmm_plan:
+            lp = self._layer_plan = _plans.LayerPlan(cg_plan, wmm_plan)
+        return lp
 
     def forward(self, fs, straight_output=False):
         if self.fused:
             if isinstance(fs, (list, tuple)):
-                B = fs[0].shape[0]
-                assert fs[0].is_cuda
-                fs = torch.cat([v.reshape(B, -1, 2) for v in fs], dim=1)
+                fs = _straight(fs)
             assert fs.is_cuda
             bn = self.bnWMM
-            new_fs = _CGBN_fused.apply(fs, bn.W, self.cg.native_plan(), bn.native_plan(), self.cg.CGspace,
-                                       bn.bn_stds, bn.bn_cnt, bn._eps_host, bn.training, self.fused_backward)
+            new_fs = _CGBN_fused.apply(fs, bn.W, self.native_layer_plan(), self.cg.CGspace, bn.bn_stds, bn.bn_cnt,
+                                       bn._eps_host, bn.training, self.fused_backward)
             if bn.batchnorm and bn.training:
                 bn.bn_cnt += 1
         else:

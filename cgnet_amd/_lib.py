@@ -43,10 +43,17 @@ SIGNATURES = {
     "cgnet_FN_WMM_backward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_FN_WMM_backward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                              ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
-    "cgnet_CGBN_backward_fused_supported": (ctypes.c_int, [_vp, _vp]),
-    "cgnet_CGBN_backward_fused_workspace": (ctypes.c_size_t, [_vp, _vp, ctypes.c_int]),
-    "cgnet_CGBN_backward_fused": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
-                                                 ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_layer_plan_create": (ctypes.c_int, [ctypes.POINTER(_vp), _vp, _vp]),
+    "cgnet_layer_plan_destroy": (ctypes.c_int, [_vp]),
+    "cgnet_CGBN_backward_fused_supported": (ctypes.c_int, [_vp]),
+    "cgnet_CGBN_backward_fused_reason": (ctypes.c_char_p, [_vp]),
+    "cgnet_CGBN_saved_bytes": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_forward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_forward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
+                                          ctypes.c_float, ctypes.c_int, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_CGBN_backward_fused_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_backward_fused": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
+                                                 ctypes.c_int, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp]),
     "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_forward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_backward_groups": (ctypes.c_int, [_vp]),

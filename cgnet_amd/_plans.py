@@ -219,28 +219,73 @@ class WMMPlan:
                                                  _stream(FF.device)))
 
 
-def fused_backward_supported(cg_plan, wmm_plan):
-    """Whether ``fused_backward`` takes this pair of plans (see cgnet_CGBN_backward_fused_supported)."""
-    return bool(_lib.load().cgnet_CGBN_backward_fused_supported(cg_plan._h, wmm_plan._h))
+class LayerPlan:
+    """One CGBN layer (``cgnet_layer_plan``): a product plan linked with the mixing plan that consumes its
+    output.  Keeps both alive.  ``fused_backward_supported`` says whether ``backward_fused`` takes the layer."""
 
+    def __init__(self, cg_plan, wmm_plan):
+        self.cg_plan, self.wmm_plan = cg_plan, wmm_plan
+        lib = _lib.load()
+        h = ctypes.c_void_p()
+        _lib.check(lib.cgnet_layer_plan_create(ctypes.byref(h), cg_plan._h, wmm_plan._h))
+        self._h = h
+        self.fused_backward_supported = bool(lib.cgnet_CGBN_backward_fused_supported(self._h))
+        self.fused_backward_reason = lib.cgnet_CGBN_backward_fused_reason(self._h).decode("utf-8", "replace")
 
-def fused_backward(cg_plan, wmm_plan, F, gF, gO, W, CG, B, stds, eps, flags):
-    """gF of the whole layer straight from gO (no gFF in memory): cgnet_CGBN_backward_fused."""
-    _require_gpu("input", F)
-    _require_gpu("grad_in", gF)
-    _require_gpu("grad_out", gO)
-    _require_gpu("W", W)
-    _require_gpu("CG", CG)
-    if flags & _lib.FN_BATCHNORM:
-        _require_gpu("FN_stds", stds)
-    else:
-        stds = None
-    if (F.numel() != B * cg_plan.nF * 2 or gF.numel() != F.numel() or gO.numel() != B * wmm_plan.nO * 2
-            or W.numel() != wmm_plan.nW * 2 or CG.numel() < cg_plan.cg_len):
-        raise RuntimeError("fused backward: tensor sizes do not match the plans")
-    lib = _lib.load()
-    with torch.cuda.device(F.device):
-        ws = _workspace(lib.cgnet_CGBN_backward_fused_workspace(cg_plan._h, wmm_plan._h, int(B)), F.device)
-        _lib.check(lib.cgnet_CGBN_backward_fused(cg_plan._h, wmm_plan._h, _ptr(F), _ptr(gF), _ptr(gO), _ptr(W), _ptr(CG),
-                                                 int(B), _ptr(stds), float(eps), int(flags), _ptr(ws), ws.numel(),
-                                                 _stream(F.device)))
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h is not None and _lib._lib is not None:
+            _lib._lib.cgnet_layer_plan_destroy(h)
+
+    def forward(self, F, FF, O, W, CG, B, stds, cnt, eps, flags, save=True):
+        """O = layer(F); FF is written too.  Returns the saved-operand tensor for ``backward_fused`` (None when
+        ``save`` is false or the fused backward is not supported)."""
+        cg, wmm = self.cg_plan, self.wmm_plan
+        cg._check_io(F, B)
+        _require_gpu("FF", FF)
+        _require_gpu("output", O)
+        _require_gpu("W", W)
+        _require_gpu("CG", CG)
+        if flags & _lib.FN_BATCHNORM:
+            _require_gpu("FN_stds", stds)
+            if stds.numel() != wmm.sum_tFF:
+                raise RuntimeError("FN_stds has %d entries, expected %d" % (stds.numel(), wmm.sum_tFF))
+        else:
+            stds = None
+        if (FF.numel() != B * cg.nFF * 2 or O.numel() != B * wmm.nO * 2 or W.numel() != wmm.nW * 2
+                or CG.numel() < cg.cg_len):
+            raise RuntimeError("CGBN forward: tensor sizes do not match the plans")
+        lib = _lib.load()
+        with torch.cuda.device(F.device):
+            saved = None
+            if save and self.fused_backward_supported:
+                saved = _workspace(lib.cgnet_CGBN_saved_bytes(self._h, int(B)), F.device)
+            ws = _workspace(lib.cgnet_CGBN_forward_workspace(self._h, int(B)), F.device)
+            _lib.check(lib.cgnet_CGBN_forward(self._h, _ptr(F), _ptr(FF), _ptr(O), _ptr(W), _ptr(CG), int(B), _ptr(stds),
+                                              float(cnt), float(eps), int(flags), _ptr(saved),
+                                              0 if saved is None else saved.numel(), _ptr(ws), ws.numel(),
+                                              _stream(F.device)))
+        return saved
+
+    def backward_fused(self, F, gF, gO, W, CG, B, stds, eps, flags, saved=None):
+        """gF of the whole layer straight from gO (no gFF in memory): cgnet_CGBN_backward_fused."""
+        cg, wmm = self.cg_plan, self.wmm_plan
+        _require_gpu("input", F)
+        _require_gpu("grad_in", gF)
+        _require_gpu("grad_out", gO)
+        _require_gpu("W", W)
+        _require_gpu("CG", CG)
+        if flags & _lib.FN_BATCHNORM:
+            _require_gpu("FN_stds", stds)
+        else:
+            stds = None
+        if (F.numel() != B * cg.nF * 2 or gF.numel() != F.numel() or gO.numel() != B * wmm.nO * 2
+                or W.numel() != wmm.nW * 2 or CG.numel() < cg.cg_len):
+            raise RuntimeError("fused backward: tensor sizes do not match the plans")
+        lib = _lib.load()
+        with torch.cuda.device(F.device):
+            ws = _workspace(lib.cgnet_CGBN_backward_fused_workspace(self._h, int(B)), F.device)
+            _lib.check(lib.cgnet_CGBN_backward_fused(self._h, _ptr(F), _ptr(gF), _ptr(gO), _ptr(W), _ptr(CG), int(B),
+                                                     _ptr(stds), float(eps), int(flags), _ptr(saved),
+                                                     0 if saved is None else saved.numel(), _ptr(ws), ws.numel(),
+                                                     _stream(F.device)))

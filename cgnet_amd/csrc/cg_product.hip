@@ -23,119 +23,7 @@
 #include <mutex>
 #include <vector>
 
-#include "common.h"
-
-namespace cgnet {
-
-struct CgTask {
-    int l, l1, l2;
-    int tau1, tau2;
-    int t1_begin, rows;   // range of t1 handled by this task
-    int offF1;            // complex offset inside a sample's F of row t1_begin of degree l1
-    int offF2;            // complex offset inside a sample's F of degree l2
-    int offFF;            // complex offset inside a sample's FF of the tile
-    int cg_off;           // float offset of the triple's table
-    int chan0;            // index over all mid channels (all degrees) of the tile's first channel
-    int nT1, nT2, TI, TJ; // forward register tiling: rows = nT1 x TI (strided), tau2 = nT2 x TJ
-    int bTI[2], bRW[2];   // backward, per slot: output channels per thread, lanes sharing one output
-};
-
-// Backward, register-resident scheme: one work-group per (sample, unit), a unit being the
-// triples that share l1 restricted to a range of t1 rows.
-struct BwdUnit {
-    int l1, rows;
-    int offF1;                // complex offset inside a sample's F of the unit's first row
-    int offF1p;               // the same inside a sample's padded fragments (rows of 2*l1+2 entries)
-    int task_begin, task_end; // range in the unit-ordered task array (sorted by l2, then l)
-    int nA;                   // waves that take slot 1; the other waves of the group take slot 2
-    int TI, RW;               // slot-1 tiling: output rows per thread, lanes sharing one output
-    int RM;                   // of those RW lanes, RM (1 or 2) split the reduced m range, RW / RM the reduced channels
-    int p1off;                // slot-1 result: -1 = the unit's rows in the slot-1 area, else offset of its rows in the
-                              // slot-2 partial area (a degree whose task list is split over several units)
-};
-
-struct BwdUTask {
-    int l, l2, tau2;
-    int offFF;                // complex offset inside a sample's gFF of the tile
-    int offF2;                // complex offset inside a sample's F of degree l2
-    int offF2p;               // the same inside a sample's padded fragments
-    int cg_off;
-    int cgp_off, cgp_len;     // float offset / length (multiple of 4) of the triple's zero-padded table
-    int p2off;                // complex offset inside a sample's slot-2 partial area of this (unit, l2) slab
-    int first_of_l2, last_of_l2;
-    int TI, RW;               // slot-2 tiling for this run of equal l2
-};
-
-// Fused layer backward, packing kernels: what packing a task's weights needs to know (one entry per BwdUTask).
-struct GenTask {
-    int aoff;                 // float offset of the task's block in the packed conj(W)/div operand
-    int nks;                  // k-steps of 4 over (output channel, re/im); 0 for a degree without output channels
-    int tO;                   // output channels of degree l
-    int chan0, nch;           // the tile's channels inside degree l: first, count (rows * tau2)
-    int cumW, K, cumT;        // degree l: complex offset of its weights, mid channels, first mid channel among all
-};
-
-// Fused layer backward, main kernel: everything a stage needs to know of its task, 12 ints that a wave reads
-// with scalar loads one stage ahead.
-struct FusedTask {
-    int geom;                 // l | l2 << 8 | tau2 << 16 | first_of_l2 << 24 | last_of_l2 << 25
-    int offF2p;               // complex offset of degree l2 inside a sample's padded fragments
-    int cgp_off, cgp_len;     // the triple's zero-padded table (floats)
-    int p2off;                // complex offset of the (unit, l2) slab in a sample's slot-2 partial area
-    int aoff;                 // float offset of the task's packed A operand
-    int shape;                // nks | tO << 8 | nch << 16
-    int boff;                 // float offset inside a sample's packed B operand of degree l
-    int chunks;               // 16-byte pieces: A block | B block << 16
-    int pad[3];
-};
-
-}  // namespace cgnet
-
-struct cgnet_cg_plan {
-    int L = 0, nllls = 0;
-    int nF = 0, nFF = 0, sumT = 0, cg_len = 0;
-    std::vector<int> t_F, t_FF, t_off, cumF, cumFF, cumT;
-    std::vector<cgnet::CgTask> fwd_tasks, bwd_tasks;
-    std::vector<int> bwd_group_begin;            // task index ranges of the backward groups (max grouping)
-    cgnet::CgTask* d_fwd_tasks = nullptr;
-    cgnet::CgTask* d_bwd_tasks = nullptr;
-    std::vector<int> bwd_group_table_off;        // for ng groups: first entry of its ng+1 boundaries
-    int* d_bwd_group_table = nullptr;
-    size_t fwd_lds = 0, bwd_lds = 0;
-    bool fwd_mm = false;                         // the forward runs cg_forward_mm_kernel (product on the matrix cores)
-    bool bwd_general_ok = true;                  // cg_backward_kernel's LDS need fits (else only the unit kernels serve)
-    std::vector<int> fwd_class_begin;            // forward tasks by LDS class: class k = tasks [begin[k], begin[k+1])
-    std::vector<size_t> fwd_class_lds;           // LDS bytes of a work-group of class k
-    int bwd_threads = 256;                       // work-group size of the backward kernel
-    // register-resident backward (used when every unit fits; otherwise the LDS-accumulator kernel)
-    bool bwd_fast = false;
-    bool bwd_hybrid = false;                     // units run cg_backward_hybrid_kernel (slot 2 on the matrix cores)
-    int bwd_hyb_groups = 0;                      // ... with this many work-groups per compute unit (4, 3 or 2)
-    std::vector<cgnet::BwdUnit> bwd_units;
-    std::vector<cgnet::BwdUTask> bwd_utasks;
-    cgnet::BwdUnit* d_bwd_units = nullptr;
-    cgnet::BwdUTask* d_bwd_utasks = nullptr;
-    int* d_bwd_combine = nullptr;                // [L+2] cumF | [L+1] own1 | [L+2] list begin | list of slab offsets
-    int* d_bwd_padmeta = nullptr;                // [L+2] cumF | [L+2] cumFp | per triple {cg_off, cgp_off, cgp_len, M, M2}
-    int bwd_nFp = 0;                             // complex entries of one sample's padded fragments
-    int bwd_cgp_len = 0;                         // floats of all padded tables
-    int bwd_f1cap = 0, bwd_f2cap = 0, bwd_cgcap = 0, bwd_tcap = 0;   // LDS bytes of the staged operands
-    int bwd_P2 = 0;                              // complex entries of one sample's slot-2 partial area
-    size_t bwd_fast_lds = 0;
-    int device = 0;
-    // fused layer backward: per-task metadata for the mixing plan this plan was linked with last (rebuilt when the
-    // signature -- t_O and the offsets per degree -- changes)
-    mutable std::mutex fused_mu;
-    mutable std::vector<int> fused_signature;
-    mutable cgnet::GenTask* d_gens = nullptr;
-    mutable cgnet::FusedTask* d_ftasks = nullptr;
-    mutable int* d_packmap = nullptr;            // per block of the weight-packing kernel: (task, row tile)
-    mutable int* d_bmap = nullptr;               // per block of the gO-packing kernel: cumO, M, t_O, column tile | k-step << 8
-    mutable int fused_npack = 0, fused_nbmap = 0;
-    mutable size_t fused_operand_floats = 0;     // packed A operand, all tasks
-    mutable int fused_bop_floats = 0;            // packed B operand of one sample
-    mutable int fused_bcap = 0, fused_acap = 0;  // LDS bytes of the B / A operand buffers
-};
+#include "internal.h"
 
 namespace cgnet {
 namespace {
@@ -831,10 +719,6 @@ __device__ __forceinline__ void bwd_item(int item, int nT, int nWin, int& w, int
     w = (widx & 1) ? c + ((widx + 1) >> 1) : c - (widx >> 1);
 }
 constexpr int kBwdMaxTI = 4;   // output channels per thread
-// Zero rows before / after the staged CG table.  The two m outputs of a thread and the two-step
-// unrolled loop touch table rows -1 .. M+1; there the coefficient is zero, so whatever finite
-// value the tile holds at the matching position (the neighbouring channel) does not count.
-constexpr int kTabLo = 1, kTabHi = 2;
 
 // Adds one task's contribution to the calling thread's accumulators.  Same arithmetic and item
 // layout as bwd_phase, one item per thread (rtid = thread index inside its role), no reduction.
@@ -1736,32 +1620,11 @@ cgbn_backward_fused_kernel(const float2* __restrict__ Fp, const float* __restric
     }
 }
 
-// The A operand of the fused kernel, one block per task, k-steps in pairs (nkp = (nks+1)/2 pairs, an odd last one
-// padded with zeros): float2 entry [(row tile * nkp + kp) * 64 + lane] = (A[c][4(2kp) + kk], A[c][4(2kp+1) + kk]) for
-// c = chan0 + 16 * row tile + lane % 16, kk = lane / 16; rows past the tile's last channel and k past 2 t_O are
-// zero.  One work-group of 64 threads per (task, row tile).
+// The A operand of the fused kernel (layout: pack_w_gen_lane), one work-group of 64 threads per (task, row tile).
 __global__ void __launch_bounds__(64)
 pack_w_gen_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                   const GenTask* __restrict__ gens, const int* __restrict__ map, float* __restrict__ Ag) {
-    const GenTask g = gens[map[2 * blockIdx.x]];
-    const int rt = map[2 * blockIdx.x + 1];
-    const int lane = threadIdx.x, i = lane & 15, kk = lane >> 4;
-    const int cl = 16 * rt + i;
-    const bool on = cl < g.nch;
-    const int c = g.chan0 + cl;
-    const int nkp = (g.nks + 1) >> 1;
-    float* dst = Ag + g.aoff + ((size_t)rt * nkp * 64 + lane) * 2;       // float2 entry [(rt * nkp + kp) * 64 + lane]
-    const float r = (on && stds) ? fmaxf(eps, stds[g.cumT + c]) : 1.f;
-    for (int ks = 0; ks < 2 * nkp; ++ks) {
-        const int k = 4 * ks + kk, to = k >> 1;
-        float v = 0.f;
-        if (on && ks < g.nks && to < g.tO) {
-            const float2 w = W[g.cumW + (size_t)to * g.K + c];
-            v = (k & 1) ? w.y : w.x;
-            if (stds) v = v / r;
-        }
-        dst[(size_t)(ks >> 1) * 128 + (ks & 1)] = v;
-    }
+    pack_w_gen_lane(W, stds, eps, gens[map[2 * blockIdx.x]], map[2 * blockIdx.x + 1], threadIdx.x, Ag);
 }
 
 // The B operand of the fused kernel, per sample and degree: entry [(column tile * nks + ks) * 64 + lane] =
@@ -1791,27 +1654,8 @@ cg_backward_pad_kernel(const float2* __restrict__ F, const float* __restrict__ C
                        float* __restrict__ CGP, const int* __restrict__ meta, int L, int nF, int nFp, int B,
                        int nbF) {
     __shared__ int s_tab[kMaxLookup];
-    const int* cumF = meta;                 // L+2
-    const int* cumFp = meta + (L + 2);      // L+2
-    const int* tri = cumFp + (L + 2);       // 5 per triple
-    if ((int)blockIdx.x < nbF) {
-        const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-        const int b = (int)(idx / nFp), e = (int)(idx % nFp);
-        const int lam = lookup_in_group(L + 1, e, [&](int k) { return cumFp[k]; }, s_tab);
-        if (idx >= (size_t)B * nFp) return;
-        const int rel = e - cumFp[lam], Mq = 2 * lam + 2;
-        const int t = rel / Mq, x = rel - t * Mq;
-        float2 v = make_float2(0.f, 0.f);
-        if (x < Mq - 1) v = F[(size_t)b * nF + cumF[lam] + t * (Mq - 1) + x];
-        Fp[idx] = v;
-    } else {
-        const int* m = tri + 5 * ((int)blockIdx.x - nbF);
-        const int cg_off = m[0], cgp_off = m[1], len = m[2], M = m[3], M2 = m[4];
-        for (int e = threadIdx.x; e < len; e += blockDim.x) {
-            const int x = e - kTabLo * M2;
-            CGP[cgp_off + e] = (x >= 0 && x < M * M2) ? CG[cg_off + x] : 0.f;
-        }
-    }
+    if ((int)blockIdx.x < nbF) pad_fragments_block(F, Fp, meta, L, nF, nFp, B, (int)blockIdx.x, s_tab);
+    else pad_table_block(CG, CGP, meta + 2 * (L + 2) + 5 * ((int)blockIdx.x - nbF));
 }
 
 // gF[b][e] = slot-1 part (if any unit owns the degree) + the slot-2 slabs of that degree, in list order
@@ -1892,13 +1736,6 @@ void* resolve_static_scratch() {
     return g_scratch_ptr[device];
 }
 
-int samples_per_group_for(int B, int ntasks) {
-    // enough work-groups to fill 256 CUs a few times over, while each group amortises the
-    // staging of its CG table over several samples
-    int groups = std::max(1, std::min(B, (6144 + ntasks - 1) / std::max(1, ntasks)));
-    return (B + groups - 1) / groups;
-}
-
 int bwd_groups_for(const cgnet_cg_plan* p, int B) {
     const int maxg = (int)p->bwd_group_begin.size() - 1;
     if (maxg <= 0) return 0;
@@ -1907,6 +1744,13 @@ int bwd_groups_for(const cgnet_cg_plan* p, int B) {
 }
 
 }  // namespace
+
+int samples_per_group_for(int B, int ntasks) {
+    // enough work-groups to fill 256 CUs a few times over, while each group amortises the
+    // staging of its CG table over several samples
+    int groups = std::max(1, std::min(B, (6144 + ntasks - 1) / std::max(1, ntasks)));
+    return (B + groups - 1) / groups;
+}
 }  // namespace cgnet
 
 using namespace cgnet;
@@ -1920,10 +1764,6 @@ static void free_plan(cgnet_cg_plan* plan) {
     if (plan->d_bwd_utasks) (void)hipFree(plan->d_bwd_utasks);
     if (plan->d_bwd_combine) (void)hipFree(plan->d_bwd_combine);
     if (plan->d_bwd_padmeta) (void)hipFree(plan->d_bwd_padmeta);
-    if (plan->d_gens) (void)hipFree(plan->d_gens);
-    if (plan->d_ftasks) (void)hipFree(plan->d_ftasks);
-    if (plan->d_packmap) (void)hipFree(plan->d_packmap);
-    if (plan->d_bmap) (void)hipFree(plan->d_bmap);
     delete plan;
 }
 
@@ -2499,7 +2339,7 @@ extern "C" int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, in
     return CGNET_OK;
 }
 
-static int launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF, const float* d_CG, int B,
+int cgnet::cg_launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF, const float* d_CG, int B,
                           double* d_part, int spg, hipStream_t s) {
     const int ntasks = (int)p->fwd_tasks.size();
     if (ntasks == 0 || B == 0) return CGNET_OK;
@@ -2530,7 +2370,7 @@ extern "C" int cgnet_sparse_forward(const cgnet_cg_plan* plan, const float* d_F,
     if (B == 0 || plan->nFF == 0) return CGNET_OK;
     CGNET_REQUIRE(d_F && d_FF && d_CG, CGNET_ERR_ARG, "null device pointer");
     const int spg = samples_per_group_for(B, (int)plan->fwd_tasks.size());
-    return launch_forward(plan, d_F, d_FF, d_CG, B, nullptr, spg, (hipStream_t)stream);
+    return cg_launch_forward(plan, d_F, d_FF, d_CG, B, nullptr, spg, (hipStream_t)stream);
 }
 
 extern "C" size_t cgnet_sparse_forward_stats_workspace(const cgnet_cg_plan* plan, int B) {
@@ -2562,7 +2402,7 @@ extern "C" int cgnet_sparse_forward_stats(const cgnet_cg_plan* plan, const float
                   "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     const int spg = samples_per_group_for(B, (int)plan->fwd_tasks.size());
     const int ngroups = (B + spg - 1) / spg;
-    int rc = launch_forward(plan, d_F, d_FF, d_CG, B, (double*)d_workspace, spg, s);
+    int rc = cg_launch_forward(plan, d_F, d_FF, d_CG, B, (double*)d_workspace, spg, s);
     if (rc != CGNET_OK) return rc;
     const int n2 = 2 * plan->sumT;
     CGNET_LAUNCH(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s,
@@ -2599,7 +2439,7 @@ extern "C" int cgnet_sparse_forward_stats_static(const cgnet_cg_plan* plan, cons
     const int ngroups = (B + spg - 1) / spg;
     // every partial sum [group][channel][2] of this call is written by the product kernel before the
     // reduction reads it, so what an earlier call left in the area needs no clearing
-    int rc = launch_forward(plan, d_F, d_FF, d_CG, B, (double*)area, spg, s);
+    int rc = cg_launch_forward(plan, d_F, d_FF, d_CG, B, (double*)area, spg, s);
     if (rc != CGNET_OK) return rc;
     CGNET_LAUNCH(stats_reduce_kernel, dim3((n2 + 255) / 256), dim3(256), 0, s, (const double*)area, d_sums, n2, ngroups);
     CGNET_HIP(hipGetLastError());
@@ -2698,25 +2538,29 @@ extern "C" int cgnet_sparse_backward(const cgnet_cg_plan* plan, const float* d_F
 }
 
 // ---- fused layer backward: host side -----------------------------------------------------------
-// Links the product plan with a mixing plan: per-task metadata on the device, rebuilt only when the mixing
-// plan's per-degree layout differs from the one linked last.  Returns CGNET_ERR_UNSUPPORTED (with the reason) for
-// shapes the fused kernel does not take.
-static int link_fused(const cgnet_cg_plan* p, const cgnet_wmm_plan* w) {
-    CGNET_REQUIRE(p->bwd_fast && p->bwd_hybrid, CGNET_ERR_UNSUPPORTED,
-                  "the fused backward needs the matrix-core unit backward (every channel count in 8..16, lmax <= 23)");
-    CGNET_REQUIRE(wmm_gradff_operand_ok(w), CGNET_ERR_UNSUPPORTED, "the fused backward needs t_O <= 16 in every degree");
+namespace cgnet {
+
+void free_fused_link(FusedLink* link) {
+    if (!link) return;
+    void* ptrs[] = {link->d_gens, link->d_ftasks, link->d_packmap, link->d_bmap};
+    for (void* q : ptrs)
+        if (q) (void)hipFree(q);
+    *link = FusedLink();
+}
+
+int build_fused_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FusedLink* link) {
+    *link = FusedLink();
     CGNET_REQUIRE(wmm_plan_degrees(w) == p->L + 1, CGNET_ERR_ARG, "the two plans have different lmax");
-    std::vector<int> sig;
     std::vector<WmmDegInfo> info(p->L + 1);
     for (int l = 0; l <= p->L; ++l) {
         if (int rc = wmm_plan_degree(w, l, &info[l])) return rc;
         CGNET_REQUIRE(info[l].K == p->t_FF[l], CGNET_ERR_ARG,
                       "degree %d: the mixing plan has %d mid channels, the product %d", l, info[l].K, p->t_FF[l]);
-        const int v[4] = {info[l].tO, info[l].cumO, info[l].cumW, info[l].cumT};
-        sig.insert(sig.end(), v, v + 4);
     }
-    std::lock_guard<std::mutex> lock(p->fused_mu);
-    if (p->d_gens && sig == p->fused_signature) return CGNET_OK;
+    link->nO = info[p->L].cumO + info[p->L].tO * (2 * p->L + 1);
+    CGNET_REQUIRE(p->bwd_fast && p->bwd_hybrid, CGNET_ERR_UNSUPPORTED,
+                  "the fused backward needs the matrix-core unit backward (every channel count in 8..16, lmax <= 23)");
+    CGNET_REQUIRE(wmm_gradff_operand_ok(w), CGNET_ERR_UNSUPPORTED, "the fused backward needs t_O <= 16 in every degree");
     // packed B operand of one sample: per degree nct x nks blocks of 64 floats
     std::vector<int> boff(p->L + 1, 0), bmap;
     int bop = 0, bcap = 16;
@@ -2774,108 +2618,88 @@ static int link_fused(const cgnet_cg_plan* p, const cgnet_wmm_plan* w) {
     const size_t lds = bwd_fused_lds(p->bwd_f1cap, p->bwd_f2cap, p->bwd_cgcap, p->bwd_tcap, bcap, acap);
     CGNET_REQUIRE(lds <= kMaxHybLds, CGNET_ERR_UNSUPPORTED,
                   "the fused backward would need %zu bytes of LDS per work-group (limit %zu)", lds, kMaxHybLds);
-    // synchronous copies: kernels of an earlier call that still read the old entries have finished when they return
-    CGNET_HIP(hipDeviceSynchronize());
+    FusedLink tmp;
     auto upload = [](const void* src, size_t bytes, void** dst) -> int {
-        if (*dst) { (void)hipFree(*dst); *dst = nullptr; }
         if (bytes == 0) return CGNET_OK;
         CGNET_HIP(hipMalloc(dst, bytes));
         CGNET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
         return CGNET_OK;
     };
-    if (int rc = upload(gens.data(), sizeof(GenTask) * gens.size(), (void**)&p->d_gens)) return rc;
-    if (int rc = upload(ft.data(), sizeof(FusedTask) * ft.size(), (void**)&p->d_ftasks)) return rc;
-    if (int rc = upload(map.data(), sizeof(int) * map.size(), (void**)&p->d_packmap)) return rc;
-    if (int rc = upload(bmap.data(), sizeof(int) * bmap.size(), (void**)&p->d_bmap)) return rc;
-    p->fused_npack = (int)(map.size() / 2);
-    p->fused_nbmap = (int)(bmap.size() / 4);
-    p->fused_operand_floats = aoff;
-    p->fused_bop_floats = bop;
-    p->fused_signature = sig;
-    p->fused_bcap = bcap;
-    p->fused_acap = acap;
-    if (int rc = raise_dynamic_lds((const void*)cgbn_backward_fused_kernel, lds)) return rc;
+    int rc = upload(gens.data(), sizeof(GenTask) * gens.size(), (void**)&tmp.d_gens);
+    if (!rc) rc = upload(ft.data(), sizeof(FusedTask) * ft.size(), (void**)&tmp.d_ftasks);
+    if (!rc) rc = upload(map.data(), sizeof(int) * map.size(), (void**)&tmp.d_packmap);
+    if (!rc) rc = upload(bmap.data(), sizeof(int) * bmap.size(), (void**)&tmp.d_bmap);
+    if (!rc) rc = raise_dynamic_lds((const void*)cgbn_backward_fused_kernel, lds);
+    if (rc) {
+        free_fused_link(&tmp);
+        return rc;
+    }
+    tmp.npack = (int)(map.size() / 2);
+    tmp.nbmap = (int)(bmap.size() / 4);
+    tmp.operand_floats = aoff;
+    tmp.bop_floats = bop;
+    tmp.bcap = bcap;
+    tmp.acap = acap;
+    tmp.nO = link->nO;
+    tmp.lds = lds;
+    tmp.ok = true;
+    *link = tmp;
     return CGNET_OK;
 }
 
-extern "C" int cgnet_CGBN_backward_fused_supported(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan) {
-    clear_error();
-    if (!cg_plan || !wmm_plan) return 0;
-    return link_fused(cg_plan, wmm_plan) == CGNET_OK ? 1 : 0;
+BwdAreas bwd_areas(const cgnet_cg_plan* p, int B) {
+    BwdAreas a{};
+    size_t o = 0;
+    a.part1 = o; o += align_up(sizeof(float) * 2 * (size_t)p->nF * B, 256);
+    a.part2 = o; o += align_up(sizeof(float) * 2 * (size_t)p->bwd_P2 * B, 256);
+    a.Fp = o;    o += align_up(sizeof(float) * 2 * (size_t)p->bwd_nFp * B, 256);
+    a.CGP = o;   o += align_up(sizeof(float) * (size_t)p->bwd_cgp_len, 256);
+    a.total = o;
+    return a;
 }
 
-static size_t fused_workspace_parts(const cgnet_cg_plan* p, int B, size_t* a_off, size_t* b_off) {
-    size_t o = cgnet_sparse_backward_workspace(p, B);
-    *a_off = o;
-    o += align_up(sizeof(float) * p->fused_operand_floats, 256);
-    *b_off = o;
-    o += align_up(sizeof(float) * (size_t)p->fused_bop_floats * B, 256);
-    return o;
-}
-
-extern "C" size_t cgnet_CGBN_backward_fused_workspace(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, int B) {
-    if (!cg_plan || !wmm_plan || B <= 0 || !cg_plan->bwd_fast) return 0;
-    if (link_fused(cg_plan, wmm_plan) != CGNET_OK) return 0;
-    size_t a, b;
-    return fused_workspace_parts(cg_plan, B, &a, &b);
-}
-
-extern "C" int cgnet_CGBN_backward_fused(const cgnet_cg_plan* plan, const cgnet_wmm_plan* wmm_plan, const float* d_F,
-                                         float* d_gF, const float* d_gO, const float* d_W, const float* d_CG, int B,
-                                         const float* d_stds, float eps, int flags, void* d_workspace,
-                                         size_t workspace_bytes, void* stream) {
-    clear_error();
-    CGNET_REQUIRE(plan && wmm_plan, CGNET_ERR_ARG, "plan is NULL");
-    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
-    if (B == 0 || plan->nF == 0) return CGNET_OK;
-    if (int rc = link_fused(plan, wmm_plan)) return rc;
-    const bool bn = flags & CGNET_FN_BATCHNORM;
-    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
-    CGNET_REQUIRE(d_F && d_gF && d_gO && d_W && d_CG, CGNET_ERR_ARG, "null device pointer");
-    CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
-    size_t a_off, b_off;
-    const size_t need = fused_workspace_parts(plan, B, &a_off, &b_off);
-    CGNET_REQUIRE(d_workspace && workspace_bytes >= need, CGNET_ERR_WORKSPACE,
-                  "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
-    CGNET_REQUIRE(((uintptr_t)d_workspace & 15) == 0, CGNET_ERR_ARG, "workspace must be 16-byte aligned");
-    hipStream_t s = (hipStream_t)stream;
-    float2* part1 = (float2*)d_workspace;
-    float2* part2 = (float2*)((char*)part1 + align_up(sizeof(float) * 2 * (size_t)plan->nF * B, 256));
-    float2* Fp = (float2*)((char*)part2 + align_up(sizeof(float) * 2 * (size_t)plan->bwd_P2 * B, 256));
-    float* CGP = (float*)((char*)Fp + align_up(sizeof(float) * 2 * (size_t)plan->bwd_nFp * B, 256));
-    float* Ag = (float*)((char*)d_workspace + a_off);
-    float* Bg = (float*)((char*)d_workspace + b_off);
-    WmmDegInfo last;
-    if (int rc = wmm_plan_degree(wmm_plan, plan->L, &last)) return rc;
-    const int nO = last.cumO + last.tO * (2 * plan->L + 1);
-    if (plan->fused_npack > 0) {
-        CGNET_LAUNCH(pack_w_gen_kernel, dim3((unsigned)plan->fused_npack), dim3(64), 0, s, (const float2*)d_W,
-                     bn ? d_stds : nullptr, eps, plan->d_gens, plan->d_packmap, Ag);
-        CGNET_HIP(hipGetLastError());
-    }
-    if (plan->fused_nbmap > 0) {
-        CGNET_LAUNCH(pack_go_gen_kernel, dim3((unsigned)plan->fused_nbmap, (unsigned)B), dim3(64), 0, s,
-                     (const float2*)d_gO, plan->d_bmap, Bg, nO, plan->fused_bop_floats);
-        CGNET_HIP(hipGetLastError());
-    }
+int launch_backward_pad(const cgnet_cg_plan* plan, const float* d_F, const float* d_CG, float* d_Fp, float* d_CGP, int B,
+                        hipStream_t s) {
     const size_t npad = (size_t)plan->bwd_nFp * B;
     const int nbF = (int)((npad + 255) / 256);
     CGNET_LAUNCH(cg_backward_pad_kernel, dim3((unsigned)(nbF + plan->nllls)), dim3(256), 0, s,
-                 (const float2*)d_F, d_CG, Fp, CGP, plan->d_bwd_padmeta, plan->L, plan->nF, plan->bwd_nFp, B, nbF);
+                 (const float2*)d_F, d_CG, (float2*)d_Fp, d_CGP, plan->d_bwd_padmeta, plan->L, plan->nF, plan->bwd_nFp, B, nbF);
     CGNET_HIP(hipGetLastError());
+    return CGNET_OK;
+}
+
+int launch_pack_w_gen(const FusedLink& link, const float* d_W, const float* d_stds, float eps, float* d_Ag, hipStream_t s) {
+    if (link.npack > 0) {
+        CGNET_LAUNCH(pack_w_gen_kernel, dim3((unsigned)link.npack), dim3(64), 0, s, (const float2*)d_W, d_stds, eps,
+                     link.d_gens, link.d_packmap, d_Ag);
+        CGNET_HIP(hipGetLastError());
+    }
+    return CGNET_OK;
+}
+
+int launch_fused_backward(const cgnet_cg_plan* plan, const FusedLink& link, const float* d_gO, const float* d_Ag,
+                          const float* d_Fp, const float* d_CGP, float* d_Bg, float* d_part1, float* d_part2,
+                          float* d_gF, int B, hipStream_t s) {
+    CGNET_REQUIRE(link.ok, CGNET_ERR_UNSUPPORTED, "the fused backward does not take this pair of plans");
+    CGNET_REQUIRE(B <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d above 65535", B);
     CGNET_REQUIRE((long long)B * (long long)plan->bwd_units.size() < (1LL << 31), CGNET_ERR_UNSUPPORTED,
                   "%d samples x %zu units exceed the grid limit", B, plan->bwd_units.size());
-    const size_t lds = bwd_fused_lds(plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, plan->fused_bcap,
-                                     plan->fused_acap);
-    CGNET_LAUNCH(cgbn_backward_fused_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads), lds, s,
-                 (const float2*)Fp, (const float*)Bg, (const float*)Ag, (const float*)CGP, part1, part2,
-                 plan->d_bwd_units, plan->d_ftasks, plan->nF, plan->bwd_nFp, plan->fused_bop_floats, plan->bwd_P2,
-                 plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, plan->fused_bcap, plan->fused_acap, B);
+    if (link.nbmap > 0) {
+        CGNET_LAUNCH(pack_go_gen_kernel, dim3((unsigned)link.nbmap, (unsigned)B), dim3(64), 0, s,
+                     (const float2*)d_gO, link.d_bmap, d_Bg, link.nO, link.bop_floats);
+        CGNET_HIP(hipGetLastError());
+    }
+    CGNET_LAUNCH(cgbn_backward_fused_kernel, dim3((unsigned)(B * plan->bwd_units.size())), dim3(kHybThreads), link.lds, s,
+                 (const float2*)d_Fp, (const float*)d_Bg, d_Ag, d_CGP, (float2*)d_part1, (float2*)d_part2,
+                 plan->d_bwd_units, link.d_ftasks, plan->nF, plan->bwd_nFp, link.bop_floats, plan->bwd_P2,
+                 plan->bwd_f1cap, plan->bwd_f2cap, plan->bwd_cgcap, plan->bwd_tcap, link.bcap, link.acap, B);
     CGNET_HIP(hipGetLastError());
     const size_t n = (size_t)plan->nF * B;
     CGNET_LAUNCH(cg_backward_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
-                 (const float2*)part1, (const float2*)part2, (float2*)d_gF, plan->d_bwd_combine, plan->L,
+                 (const float2*)d_part1, (const float2*)d_part2, (float2*)d_gF, plan->d_bwd_combine, plan->L,
                  plan->nF, plan->bwd_P2, B);
     CGNET_HIP(hipGetLastError());
     return CGNET_OK;
 }
+
+}  // namespace cgnet

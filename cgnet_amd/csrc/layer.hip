@@ -1,0 +1,265 @@
+// One CGNet layer (CG product -> fragment norm -> weight mixing) as a unit: the link between a product plan and
+// the mixing plan that consumes its output, a forward that prepares in one launch everything the later kernels
+// read (packed weights of the mixing, and for the backward the packed weights of the fused kernel, the padded
+// fragments and the padded tables), and the entry point of the one-kernel layer backward.
+#include <algorithm>
+#include <cstring>
+#include <memory>
+
+#include "internal.h"
+
+struct cgnet_layer_plan {
+    const cgnet_cg_plan* cg = nullptr;
+    const cgnet_wmm_plan* wmm = nullptr;
+    cgnet::FusedLink link;
+    char reason[512] = "";       // why the fused backward does not take this layer ("" if it does)
+};
+
+namespace cgnet {
+namespace {
+
+// Running fragment-norm values from the per-group partial sums of the product kernel: the groups are added in
+// order (as stats_reduce_kernel does), then the moving average is updated (as fn_update_std_kernel does).
+__global__ void __launch_bounds__(256)
+fn_finish_kernel(const double* __restrict__ part, int ngroups, float* __restrict__ stds,
+                 const WmmDeg* __restrict__ degs, int ndeg, int sumT, int B, float cnt) {
+    __shared__ int s_tab[kMaxLookup];
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int di = lookup_in_group(ndeg, c, [&](int k) { return degs[k].cumT; }, s_tab);
+    if (c >= sumT) return;
+    double s1 = 0., s2 = 0.;
+    for (int g = 0; g < ngroups; ++g) {
+        const double2 v = reinterpret_cast<const double2*>(part)[(size_t)g * sumT + c];
+        s1 += v.x;
+        s2 += v.y;
+    }
+    stds[c] = updated_std(stds[c], s1, s2, (double)B * (double)degs[di].M, cnt);
+}
+
+// Everything the kernels after the statistics read that depends only on W, the (updated) stds, F and the table, in
+// one launch; the work-groups are dealt out by role:
+//   [0, nb_fwd)      packed weights of the mixing forward               (pack_w_forward_thread)
+//   [.., + nb_gen)   packed weights of the fused backward, four (task, row tile) pairs each   (pack_w_gen_lane)
+//   [.., + nbF)      fragments with a zero behind every row             (pad_fragments_block)
+//   [.., + ntab)     every triple's table between zero rows             (pad_table_block)
+__global__ void __launch_bounds__(256)
+layer_prepare_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                     const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int wp_blocks, int nb_fwd,
+                     const GenTask* __restrict__ gens, const int* __restrict__ packmap, int npack, float* __restrict__ Ag,
+                     int nb_gen, const float2* __restrict__ F, const float* __restrict__ CG, float2* __restrict__ Fp,
+                     float* __restrict__ CGP, const int* __restrict__ padmeta, int L, int nF, int nFp, int B, int nbF) {
+    __shared__ int s_tab[kMaxLookup];
+    int blk = (int)blockIdx.x;
+    if (blk < nb_fwd) {
+        pack_w_forward_thread(W, stds, eps, degs, ndeg, Wp, wp_blocks, blk * 256 + (int)threadIdx.x, s_tab);
+        return;
+    }
+    blk -= nb_fwd;
+    if (blk < nb_gen) {
+        const int pair = blk * 4 + (int)(threadIdx.x >> 6);
+        if (pair < npack) pack_w_gen_lane(W, stds, eps, gens[packmap[2 * pair]], packmap[2 * pair + 1], threadIdx.x & 63, Ag);
+        return;
+    }
+    blk -= nb_gen;
+    if (blk < nbF) {
+        pad_fragments_block(F, Fp, padmeta, L, nF, nFp, B, blk, s_tab);
+        return;
+    }
+    blk -= nbF;
+    pad_table_block(CG, CGP, padmeta + 2 * (L + 2) + 5 * blk);
+}
+
+struct SavedAreas { size_t Ag, Fp, CGP, total; };
+SavedAreas saved_areas(const cgnet_layer_plan* lp, int B) {
+    SavedAreas a{};
+    if (!lp->link.ok || B <= 0) return a;
+    size_t o = 0;
+    a.Ag = o;  o += align_up(sizeof(float) * lp->link.operand_floats, 256);
+    a.Fp = o;  o += align_up(sizeof(float) * 2 * (size_t)lp->cg->bwd_nFp * B, 256);
+    a.CGP = o; o += align_up(sizeof(float) * (size_t)lp->cg->bwd_cgp_len, 256);
+    a.total = o;
+    return a;
+}
+
+struct FwdAreas { size_t part, wp, opart, total; int spg, ngroups; };
+FwdAreas forward_areas(const cgnet_layer_plan* lp, int B) {
+    FwdAreas a{};
+    a.spg = samples_per_group_for(B, (int)lp->cg->fwd_tasks.size());
+    a.ngroups = (B + a.spg - 1) / a.spg;
+    size_t o = 0;
+    a.part = o;  o += align_up(sizeof(double) * 2 * (size_t)lp->cg->sumT * a.ngroups, 256);
+    a.wp = o;    o += align_up(wmm_forward_wp_bytes(lp->wmm), 256);
+    a.opart = o; o += align_up(wmm_forward_opart_bytes(lp->wmm, B), 256);
+    a.total = o;
+    return a;
+}
+
+struct BwdFusedAreas { BwdAreas own; size_t Ag, Bg, total; };
+BwdFusedAreas backward_areas(const cgnet_layer_plan* lp, int B) {
+    BwdFusedAreas a{};
+    a.own = bwd_areas(lp->cg, B);
+    size_t o = a.own.total;
+    a.Ag = o; o += align_up(sizeof(float) * lp->link.operand_floats, 256);
+    a.Bg = o; o += align_up(sizeof(float) * (size_t)lp->link.bop_floats * B, 256);
+    a.total = o;
+    return a;
+}
+
+}  // namespace
+}  // namespace cgnet
+
+using namespace cgnet;
+
+extern "C" int cgnet_layer_plan_create(cgnet_layer_plan** plan, const cgnet_cg_plan* cg_plan,
+                                       const cgnet_wmm_plan* wmm_plan) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    *plan = nullptr;
+    CGNET_REQUIRE(cg_plan && wmm_plan, CGNET_ERR_ARG, "null plan");
+    CGNET_REQUIRE(wmm_plan->L == cg_plan->L, CGNET_ERR_ARG, "the two plans have different lmax (%d, %d)", cg_plan->L,
+                  wmm_plan->L);
+    for (int l = 0; l <= cg_plan->L; ++l)
+        CGNET_REQUIRE(wmm_plan->degs[l].K == cg_plan->t_FF[l], CGNET_ERR_ARG,
+                      "degree %d: the mixing plan has %d mid channels, the product %d", l, wmm_plan->degs[l].K,
+                      cg_plan->t_FF[l]);
+    std::unique_ptr<cgnet_layer_plan> p(new cgnet_layer_plan());
+    p->cg = cg_plan;
+    p->wmm = wmm_plan;
+    const int rc = build_fused_link(cg_plan, wmm_plan, &p->link);
+    if (rc == CGNET_ERR_UNSUPPORTED) {
+        // the layer still runs, with the two-kernel backward
+        std::strncpy(p->reason, cgnet_last_error(), sizeof(p->reason) - 1);
+        clear_error();
+    } else if (rc != CGNET_OK) {
+        return rc;
+    }
+    *plan = p.release();
+    return CGNET_OK;
+}
+
+extern "C" int cgnet_layer_plan_destroy(cgnet_layer_plan* plan) {
+    clear_error();
+    if (!plan) return CGNET_OK;
+    free_fused_link(&plan->link);
+    delete plan;
+    return CGNET_OK;
+}
+
+extern "C" int cgnet_CGBN_backward_fused_supported(const cgnet_layer_plan* plan) {
+    return plan && plan->link.ok ? 1 : 0;
+}
+
+extern "C" const char* cgnet_CGBN_backward_fused_reason(const cgnet_layer_plan* plan) {
+    return plan ? plan->reason : "no plan";
+}
+
+extern "C" size_t cgnet_CGBN_saved_bytes(const cgnet_layer_plan* plan, int B) {
+    return plan ? saved_areas(plan, B).total : 0;
+}
+
+extern "C" size_t cgnet_CGBN_forward_workspace(const cgnet_layer_plan* plan, int B) {
+    if (!plan || B <= 0) return 0;
+    return forward_areas(plan, B).total;
+}
+
+extern "C" int cgnet_CGBN_forward(const cgnet_layer_plan* plan, const float* d_F, float* d_FF, float* d_O,
+                                  const float* d_W, const float* d_CG, int B, float* d_stds, float cnt, float eps,
+                                  int flags, void* d_saved, size_t saved_bytes, void* d_workspace,
+                                  size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    if (B == 0) return CGNET_OK;
+    const cgnet_cg_plan* cg = plan->cg;
+    const cgnet_wmm_plan* wmm = plan->wmm;
+    const bool bn = flags & CGNET_FN_BATCHNORM, upd = bn && (flags & CGNET_FN_UPDATE_STD);
+    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    CGNET_REQUIRE(cg->nF == 0 || d_F, CGNET_ERR_ARG, "d_F is NULL");
+    CGNET_REQUIRE(cg->nFF == 0 || (d_FF && d_CG), CGNET_ERR_ARG, "d_FF or d_CG is NULL");
+    CGNET_REQUIRE(wmm->nO == 0 || d_O, CGNET_ERR_ARG, "d_O is NULL");
+    CGNET_REQUIRE(wmm->nW == 0 || d_W, CGNET_ERR_ARG, "d_W is NULL");
+    const FwdAreas fa = forward_areas(plan, B);
+    CGNET_REQUIRE(d_workspace && workspace_bytes >= fa.total, CGNET_ERR_WORKSPACE,
+                  "workspace of %zu bytes given, %zu needed", workspace_bytes, fa.total);
+    const SavedAreas sa = saved_areas(plan, B);
+    const bool save = d_saved != nullptr && sa.total > 0;
+    CGNET_REQUIRE(!save || saved_bytes >= sa.total, CGNET_ERR_WORKSPACE,
+                  "saved-operand area of %zu bytes given, %zu needed", saved_bytes, sa.total);
+    CGNET_REQUIRE(!save || ((uintptr_t)d_saved & 15) == 0, CGNET_ERR_ARG, "the saved-operand area must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)d_workspace;
+    const int ndeg = (int)wmm->degs.size();
+
+    // product, with the per-group partial statistics when the running stds are to be updated
+    const bool stats = upd && cg->sumT > 0 && cg->nFF > 0;
+    if (cg->nFF > 0)
+        if (int rc = cg_launch_forward(cg, d_F, d_FF, d_CG, B, stats ? (double*)(ws + fa.part) : nullptr, fa.spg, s)) return rc;
+    if (stats) {
+        CGNET_LAUNCH(fn_finish_kernel, dim3((cg->sumT + 255) / 256), dim3(256), 0, s, (const double*)(ws + fa.part),
+                     fa.ngroups, d_stds, wmm->d_degs, ndeg, cg->sumT, B, cnt);
+        CGNET_HIP(hipGetLastError());
+    }
+    // the operands of the mixing forward and (when asked for) of the backward
+    float* Wp = (float*)(ws + fa.wp);
+    const bool pack_fwd = wmm->nO > 0 && !wmm->fwd_units.empty();
+    const int nb_fwd = pack_fwd ? (wmm->wp_blocks * 16 + 255) / 256 : 0;
+    const int nb_gen = save ? (plan->link.npack + 3) / 4 : 0;
+    const int nbF = save ? (int)(((size_t)cg->bwd_nFp * B + 255) / 256) : 0;
+    const int ntab = save ? cg->nllls : 0;
+    if (nb_fwd + nb_gen + nbF + ntab > 0) {
+        char* sv = (char*)d_saved;
+        CGNET_LAUNCH(layer_prepare_kernel, dim3((unsigned)(nb_fwd + nb_gen + nbF + ntab)), dim3(256), 0, s,
+                     (const float2*)d_W, bn ? d_stds : nullptr, eps, wmm->d_degs, ndeg, Wp, wmm->wp_blocks, nb_fwd,
+                     plan->link.d_gens, plan->link.d_packmap, plan->link.npack, save ? (float*)(sv + sa.Ag) : nullptr,
+                     nb_gen, (const float2*)d_F, d_CG, save ? (float2*)(sv + sa.Fp) : nullptr,
+                     save ? (float*)(sv + sa.CGP) : nullptr, cg->d_bwd_padmeta, cg->L, cg->nF, cg->bwd_nFp, B, nbF);
+        CGNET_HIP(hipGetLastError());
+    }
+    return wmm_forward_packed(wmm, d_FF, d_O, Wp, B, ws + fa.opart, s);
+}
+
+extern "C" size_t cgnet_CGBN_backward_fused_workspace(const cgnet_layer_plan* plan, int B) {
+    if (!plan || B <= 0 || !plan->link.ok) return 0;
+    return backward_areas(plan, B).total;
+}
+
+extern "C" int cgnet_CGBN_backward_fused(const cgnet_layer_plan* plan, const float* d_F, float* d_gF, const float* d_gO,
+                                         const float* d_W, const float* d_CG, int B, const float* d_stds, float eps,
+                                         int flags, const void* d_saved, size_t saved_bytes, void* d_workspace,
+                                         size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    const cgnet_cg_plan* cg = plan->cg;
+    if (B == 0 || cg->nF == 0) return CGNET_OK;
+    CGNET_REQUIRE(plan->link.ok, CGNET_ERR_UNSUPPORTED, "%s", plan->reason);
+    const bool bn = flags & CGNET_FN_BATCHNORM;
+    CGNET_REQUIRE(d_gF && d_gO, CGNET_ERR_ARG, "null device pointer");
+    const BwdFusedAreas ba = backward_areas(plan, B);
+    CGNET_REQUIRE(d_workspace && workspace_bytes >= ba.total, CGNET_ERR_WORKSPACE,
+                  "workspace of %zu bytes given, %zu needed", workspace_bytes, ba.total);
+    CGNET_REQUIRE(((uintptr_t)d_workspace & 15) == 0, CGNET_ERR_ARG, "workspace must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)d_workspace;
+    const float *Ag, *Fp, *CGP;
+    if (d_saved) {
+        const SavedAreas sa = saved_areas(plan, B);
+        CGNET_REQUIRE(saved_bytes >= sa.total, CGNET_ERR_WORKSPACE, "saved-operand area of %zu bytes given, %zu needed",
+                      saved_bytes, sa.total);
+        CGNET_REQUIRE(((uintptr_t)d_saved & 15) == 0, CGNET_ERR_ARG, "the saved-operand area must be 16-byte aligned");
+        const char* sv = (const char*)d_saved;
+        Ag = (const float*)(sv + sa.Ag);
+        Fp = (const float*)(sv + sa.Fp);
+        CGP = (const float*)(sv + sa.CGP);
+    } else {
+        CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+        CGNET_REQUIRE(d_F && d_W && d_CG, CGNET_ERR_ARG, "null device pointer");
+        if (int rc = launch_pack_w_gen(plan->link, d_W, bn ? d_stds : nullptr, eps, (float*)(ws + ba.Ag), s)) return rc;
+        if (int rc = launch_backward_pad(cg, d_F, d_CG, (float*)(ws + ba.own.Fp), (float*)(ws + ba.own.CGP), B, s)) return rc;
+        Ag = (const float*)(ws + ba.Ag);
+        Fp = (const float*)(ws + ba.own.Fp);
+        CGP = (const float*)(ws + ba.own.CGP);
+    }
+    return launch_fused_backward(cg, plan->link, d_gO, Ag, Fp, CGP, (float*)(ws + ba.Bg), (float*)(ws + ba.own.part1),
+                                 (float*)(ws + ba.own.part2), d_gF, B, s);
+}

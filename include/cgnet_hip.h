@@ -162,24 +162,54 @@ int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_gO, float* 
                           float eps, int flags,
                           void* d_workspace, size_t workspace_bytes, void* stream);
 
-/* ---- the whole layer's backward in one pass (no counterpart in the reference) -------------------- */
+/* ---- the layer as a unit (no counterpart in the reference) ------------------------------------------ */
 
-/* gF = dLoss/dF of  F -> CG product -> fragment norm + weight mixing -> O  from d_gO = dLoss/dO, i.e. what
- * cgnet_FN_WMM_backward(d_gFF = ...) followed by cgnet_sparse_backward(d_gFF) returns in d_gF, bit for bit,
- * without the intermediate gradient gFF (B x nFF complex) ever existing in memory: every tile of it is formed
- * in LDS on the matrix cores from gO and conj(W)/div right where the product's backward consumes it.  The
- * reference has no such call (its two autograd Functions meet at a materialised grad_FF,
- * CGNet/CG_layers.py:54-72,194-203); it is legal wherever FF is not visible to the user, i.e. inside
- * CGBN_cuda.forward (CG_layers.py:313-318).  The weight gradient still comes from cgnet_FN_WMM_backward
- * (d_gFF = NULL).  cgnet_CGBN_backward_fused_supported returns 1 for the shapes the fused kernel takes
- * (every input channel count in 8..16, lmax <= 23, t_O <= 16, LDS within limits) and 0 otherwise, with
- * cgnet_last_error() naming the reason; the call itself then returns CGNET_ERR_UNSUPPORTED.
- * d_stds / eps / flags as in cgnet_FN_WMM_backward (the stds the forward pass used, treated as constants). */
-int cgnet_CGBN_backward_fused_supported(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan);
-size_t cgnet_CGBN_backward_fused_workspace(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, int B);
-int cgnet_CGBN_backward_fused(const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan, const float* d_F,
-                              float* d_gF, const float* d_gO, const float* d_W, const float* d_CG, int B,
-                              const float* d_stds, float eps, int flags,
+/* One CGNet layer, F -> CG product -> fragment norm + weight mixing -> O (CGBN_cuda.forward, CGNet/CG_layers.py:313-318),
+ * as a unit.  The reference chains two autograd Functions that meet at the materialised tensors FF and grad_FF
+ * (CG_layers.py:14-72,168-203); inside the layer neither is visible to the user, which these entry points use:
+ * the forward prepares in one launch every operand the later kernels read, and the backward can go from gO to gF
+ * in one kernel without grad_FF in memory.
+ *
+ * A layer plan links a product plan with the mixing plan that consumes its output (t_FF must agree).  It keeps
+ * pointers to both, which must outlive it, and a little device memory of its own (allocated here, at creation, on
+ * the current device; never changed afterwards, so concurrent calls need no lock and no per-call entry point
+ * allocates). */
+typedef struct cgnet_layer_plan cgnet_layer_plan;
+int cgnet_layer_plan_create(cgnet_layer_plan** plan, const cgnet_cg_plan* cg_plan, const cgnet_wmm_plan* wmm_plan);
+int cgnet_layer_plan_destroy(cgnet_layer_plan* plan);
+
+/* 1 if cgnet_CGBN_backward_fused takes this layer (every input channel count in 8..16, lmax <= 23, t_O <= 16,
+ * LDS within limits), else 0; cgnet_CGBN_backward_fused_reason then names what is missing. */
+int cgnet_CGBN_backward_fused_supported(const cgnet_layer_plan* plan);
+const char* cgnet_CGBN_backward_fused_reason(const cgnet_layer_plan* plan);
+
+/* O = layer(F): cgnet_sparse_forward_stats (statistics only with CGNET_FN_UPDATE_STD) followed by
+ * cgnet_FN_WMM_forward(d_sums = ...), same arithmetic and same results bit for bit, in fewer launches: the
+ * statistics are reduced and the running stds updated in one kernel, and one further kernel packs the weights of
+ * the mixing and -- when d_saved is given -- the three operands cgnet_CGBN_backward_fused would otherwise build
+ * itself (packed W / max(eps, stds) per task, F with a zero behind every row, the tables between zero rows), all of
+ * which depend only on what the forward already holds.  d_FF (B x nFF complex) is written as by
+ * cgnet_sparse_forward: the weight gradient needs it.  d_saved: cgnet_CGBN_saved_bytes(plan, B) bytes, 16-byte
+ * aligned, or NULL (inference; also when the fused backward is not supported, where the size is 0).
+ * d_stds / cnt / eps / flags as in cgnet_FN_WMM_forward. */
+size_t cgnet_CGBN_saved_bytes(const cgnet_layer_plan* plan, int B);
+size_t cgnet_CGBN_forward_workspace(const cgnet_layer_plan* plan, int B);
+int cgnet_CGBN_forward(const cgnet_layer_plan* plan, const float* d_F, float* d_FF, float* d_O, const float* d_W,
+                       const float* d_CG, int B, float* d_stds, float cnt, float eps, int flags,
+                       void* d_saved, size_t saved_bytes, void* d_workspace, size_t workspace_bytes, void* stream);
+
+/* gF = dLoss/dF of the layer from d_gO = dLoss/dO, i.e. what cgnet_FN_WMM_backward(d_gFF = ...) followed by
+ * cgnet_sparse_backward(d_gFF) returns in d_gF, without the intermediate gradient gFF (B x nFF complex) ever
+ * existing in memory: every tile of it is formed in LDS on the matrix cores from gO and W / div right where the
+ * product's backward consumes it.  The weight gradient still comes from cgnet_FN_WMM_backward (d_gFF = NULL).
+ * With d_saved (the area cgnet_CGBN_forward filled for the same F, W, stds, table and B) d_F, d_W, d_CG and d_stds
+ * are not read and may be NULL; with d_saved = NULL the call builds those operands itself (two more launches).
+ * d_stds / eps / flags as in cgnet_FN_WMM_backward (the stds the forward pass used, treated as constants).
+ * Returns CGNET_ERR_UNSUPPORTED where cgnet_CGBN_backward_fused_supported is 0.  Allocates nothing. */
+size_t cgnet_CGBN_backward_fused_workspace(const cgnet_layer_plan* plan, int B);
+int cgnet_CGBN_backward_fused(const cgnet_layer_plan* plan, const float* d_F, float* d_gF, const float* d_gO,
+                              const float* d_W, const float* d_CG, int B, const float* d_stds, float eps, int flags,
+                              const void* d_saved, size_t saved_bytes,
                               void* d_workspace, size_t workspace_bytes, void* stream);
 
 /* ---- measurement hooks (no counterpart in the reference, which times nothing) ------------ */

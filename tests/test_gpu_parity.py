@@ -590,11 +590,10 @@ def test_fused_backward_equals_two_kernel_backward(dev, lmax, tin, tout, bsz, sp
     """The one-kernel backward (gFF tiles formed in LDS) returns bit for bit what the gFF kernel followed by the
     product's backward returns, for the input gradient and the weight gradient, in training mode; the small
     cases are also held against the oracle."""
-    from cgnet_amd import _plans
     mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=400 + k)
-    if not _plans.fused_backward_supported(mod.cg.native_plan(), mod.bnWMM.native_plan()):
-        from cgnet_amd import _lib
-        pytest.skip("shape not taken by the fused backward: " + _lib.load().cgnet_last_error().decode())
+    lp = mod.native_layer_plan()
+    if not lp.fused_backward_supported:
+        pytest.skip("shape not taken by the fused backward: " + lp.fused_backward_reason)
     x64 = rand_straight(tin, bsz, seed=500 + k)
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
     go = randn32((bsz, n_o, 2), torch.Generator().manual_seed(600 + k)).float().to(dev)
@@ -648,26 +647,57 @@ def test_layer_random_shapes(dev, lmax, tin, tout, bsz, sparse, bn, k):
     check_layer_step(dev, mod, ora, twin, w64, x64, go64)
 
 
-def test_layer_backward_two_streams_matches_one_stream(dev, monkeypatch):
-    """The layer's backward runs the weight gradient on a second stream; several steps back to back, without a
-    host synchronisation in between, must give bit for bit what the same steps give on one stream."""
-    from cgnet_amd import CG_layers
+def test_layer_steps_back_to_back(dev):
+    """Several training steps back to back, without a host synchronisation in between (every step reuses the
+    workspaces and saved-operand areas the caching allocator hands back), give bit for bit what the same steps
+    give with a synchronisation after every call, on both backward routes."""
     lmax, tin, tout, bsz = 6, [9, 8, 12, 10, 16, 8, 11], [8] * 7, 7
     x = rand_straight(tin, bsz, seed=31).float().to(dev)
     g = torch.Generator().manual_seed(33)
     n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
     gos = [torch.randn(bsz, n_o, 2, generator=g).to(dev) for _ in range(4)]
-    results = []
-    for overlap in (1, 0):
-        monkeypatch.setattr(CG_layers, "_OVERLAP_GRAD_W", overlap)
-        mod, _, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=7)
-        mod.train()
-        xs = x.clone().requires_grad_(True)
-        for go in gos:                                   # gradients accumulate over the steps
-            mod(xs, straight_output=True).backward(go)
-        results.append((xs.grad.clone(), mod.bnWMM.W.grad.clone(), mod.bnWMM.bn_stds.detach().clone()))
-    for a, b in zip(*results):
-        assert torch.equal(a, b)
+    for fused_backward in (True, False):
+        results = []
+        for sync in (False, True):
+            mod, _, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=7)
+            mod.fused_backward = fused_backward
+            mod.train()
+            xs = x.clone().requires_grad_(True)
+            for go in gos:                                   # gradients accumulate over the steps
+                out = mod(xs, straight_output=True)
+                if sync:
+                    torch.cuda.synchronize()
+                out.backward(go)
+                if sync:
+                    torch.cuda.synchronize()
+            results.append((xs.grad.clone(), mod.bnWMM.W.grad.clone(), mod.bnWMM.bn_stds.detach().clone()))
+        for a, b in zip(*results):
+            assert torch.equal(a, b)
+
+
+def test_fused_backward_builds_its_own_operands(dev):
+    """cgnet_CGBN_backward_fused without the operand area of the forward (d_saved = NULL) packs the weights and pads
+    the fragments and tables itself: same input gradient, bit for bit."""
+    lmax, tin, tout, bsz = 5, [9, 8, 12, 10, 16, 8], [8, 0, 5, 16, 3, 7], 3
+    mod, _, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=11)
+    lp = mod.native_layer_plan()
+    assert lp.fused_backward_supported, lp.fused_backward_reason
+    x = rand_straight(tin, bsz, seed=41).float().to(dev)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go = torch.randn(bsz, n_o, 2, generator=torch.Generator().manual_seed(43)).to(dev)
+    bn = mod.bnWMM
+    FF = torch.empty(bsz, lp.cg_plan.nFF, 2, device=dev)
+    out = torch.empty(bsz, n_o, 2, device=dev)
+    flags = 0x1 | 0x2
+    saved = lp.forward(x, FF, out, bn.W.detach(), mod.cg.CGspace, bsz, bn.bn_stds.data, 1.0, bn._eps_host, flags, save=True)
+    assert saved is not None
+    grads = []
+    for sv in (saved, None):
+        gF = torch.full_like(x, float("nan"))
+        lp.backward_fused(x, gF, go, bn.W.detach(), mod.cg.CGspace, bsz, bn.bn_stds.data, bn._eps_host, flags, sv)
+        grads.append(gF)
+    assert torch.isfinite(grads[0]).all()
+    assert torch.equal(grads[0], grads[1])
 
 
 def real_signal_coefficients(lmax, bsz, gen):
