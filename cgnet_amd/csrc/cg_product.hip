@@ -354,7 +354,6 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
             dre = mfma4(nai, fb.y, dre);
             dim = mfma4(ai, fb.x, dim);
         }
-        mfma_drain();
         if (i < tau2) {
             float2* o = out + (4 * kk * tau2 + i) * M + mm;
 #pragma unroll
@@ -1289,7 +1288,6 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         bwd_stage_end<kHybThreads, false>(c, u, ti, t);
         if (cur.last_of_l2) {
             const int M2 = 2 * cur.l2 + 1;
-            mfma_drain();
             bwd_mm_store(dre, dim, cur.tau2, M2, lane, part2_b + cur.p2off + (size_t)part * cur.tau2 * M2);
 #pragma unroll
             for (int k = 0; k < kHybMaxTiles; ++k) dre[k] = dim[k] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -1448,7 +1446,6 @@ __device__ __forceinline__ void gen_phase_nks(int nch, int M, const float* __res
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) acc = mfma4(a[ks], bv[ks], acc);
-            mfma_drain();
             const int row = 16 * rt + 4 * kk;
             float* dst = tile + row * M2f + col;
             if (16 * rt + 16 <= nch) {               // wave-uniform: a full row tile
@@ -1557,7 +1554,6 @@ __device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u
         bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, c.lane, dre, dim);
         if (ft_last(t)) {
             const int M2 = 2 * l2 + 1;
-            mfma_drain();
             bwd_mm_store(dre, dim, tau2, M2, c.lane, part2_b + t.p2off + (size_t)part * tau2 * M2);
 #pragma unroll
             for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};

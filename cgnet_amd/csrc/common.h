@@ -89,15 +89,6 @@ __device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
-// Called between the last matrix instruction of a chain and the first ordinary read of its
-// accumulators: gives the matrix pipeline time to retire its results (an accumulator read
-// hoisted directly behind the chain returned stale values otherwise).
-__device__ __forceinline__ void mfma_drain() {
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
 // ---- global memory -> LDS copies that bypass the registers (gfx950 LDS-direct loads) ----------
 // The hardware places lane i of a wave 16*i (4*i for dword copies) bytes behind the LDS address
 // the wave passes; the copy is tracked by vmcnt.  Nothing may read the destination before the

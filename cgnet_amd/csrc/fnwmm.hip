@@ -237,7 +237,6 @@ __device__ __forceinline__ void wmm_forward_wave(const float2* __restrict__ FF, 
             }
         }
     }
-    mfma_drain();
     // complex outputs: the re / im columns of a complex column sit in the same lane
     float2* dst = out + (size_t)u.slice * B * nO;
 #pragma unroll
@@ -419,14 +418,12 @@ wmm_gradw_kernel(const float2* __restrict__ gO, const float2* __restrict__ FF, f
             }
             if (++since == kGradWFold) {
                 since = 0;
-                mfma_drain();
                 tot0 += acc0;
                 tot1 += acc1;
                 acc0 = acc1 = (f32x4){0.f, 0.f, 0.f, 0.f};
             }
         }
     }
-    mfma_drain();
     tot0 += acc0;
     tot1 += acc1;
     if (cok) {
@@ -639,7 +636,6 @@ __device__ __forceinline__ void wmm_gradff_wave(const float2* __restrict__ gO, c
                     for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
                         for (int t = 0; t < NT; ++t) acc[t] = mfma4(a[sub][ks], bv[ks][t], acc[t]);
-                    mfma_drain();
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
                         const int col = (ct0 + t) * 16 + i;

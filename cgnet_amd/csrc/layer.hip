@@ -20,7 +20,7 @@ namespace {
 
 // Running fragment-norm values from the per-group partial sums of the product kernel: the groups are added in
 // order (as stats_reduce_kernel does), then the moving average is updated (as fn_update_std_kernel does).
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 fn_finish_kernel(const double* __restrict__ part, int ngroups, float* __restrict__ stds,
                  const WmmDeg* __restrict__ degs, int ndeg, int sumT, int B, float cnt) {
     __shared__ int s_tab[kMaxLookup];
@@ -28,8 +28,18 @@ fn_finish_kernel(const double* __restrict__ part, int ngroups, float* __restrict
     const int di = lookup_in_group(ndeg, c, [&](int k) { return degs[k].cumT; }, s_tab);
     if (c >= sumT) return;
     double s1 = 0., s2 = 0.;
-    for (int g = 0; g < ngroups; ++g) {
-        const double2 v = reinterpret_cast<const double2*>(part)[(size_t)g * sumT + c];
+    const double2* p = reinterpret_cast<const double2*>(part) + c;
+    int g = 0;
+    for (; g + 4 <= ngroups; g += 4) {               // four loads in flight, added in group order
+        const double2 v0 = p[(size_t)g * sumT], v1 = p[(size_t)(g + 1) * sumT];
+        const double2 v2 = p[(size_t)(g + 2) * sumT], v3 = p[(size_t)(g + 3) * sumT];
+        s1 += v0.x; s2 += v0.y;
+        s1 += v1.x; s2 += v1.y;
+        s1 += v2.x; s2 += v2.y;
+        s1 += v3.x; s2 += v3.y;
+    }
+    for (; g < ngroups; ++g) {
+        const double2 v = p[(size_t)g * sumT];
         s1 += v.x;
         s2 += v.y;
     }
@@ -195,7 +205,7 @@ extern "C" int cgnet_CGBN_forward(const cgnet_layer_plan* plan, const float* d_F
     if (cg->nFF > 0)
         if (int rc = cg_launch_forward(cg, d_F, d_FF, d_CG, B, stats ? (double*)(ws + fa.part) : nullptr, fa.spg, s)) return rc;
     if (stats) {
-        CGNET_LAUNCH(fn_finish_kernel, dim3((cg->sumT + 255) / 256), dim3(256), 0, s, (const double*)(ws + fa.part),
+        CGNET_LAUNCH(fn_finish_kernel, dim3((cg->sumT + 63) / 64), dim3(64), 0, s, (const double*)(ws + fa.part),
                      fa.ngroups, d_stds, wmm->d_degs, ndeg, cg->sumT, B, cnt);
         CGNET_HIP(hipGetLastError());
     }
