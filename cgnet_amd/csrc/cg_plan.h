@@ -54,6 +54,8 @@ struct GenTask {
     int tO;                   // output channels of degree l
     int chan0, nch;           // the tile's channels inside degree l: first, count (rows * tau2)
     int cumW, K, cumT;        // degree l: complex offset of its weights, mid channels, first mid channel among all
+    int sym;                  // 0, or +-tau for a diagonal triple with tau x tau channels: channel (t1, t2) is packed as its own
+                              // weight plus sign(sym) times that of channel (t2, t1)
 };
 
 // Fused layer backward, main kernel: everything a stage needs to know of its task, 12 ints that a wave reads
@@ -149,6 +151,14 @@ __device__ __forceinline__ void pack_w_gen_lane(const float2* __restrict__ W, co
     const int nkp = (g.nks + 1) >> 1;
     float* dst = Ag + g.aoff + ((size_t)rt * nkp * 64 + lane) * 2;       // float2 entry [(rt * nkp + kp) * 64 + lane]
     const float r = (on && stds) ? fmaxf(eps, stds[g.cumT + c]) : 1.f;
+    // the mirror channel (t2, t1) of a diagonal triple's channel (t1, t2)
+    const int tau = g.sym < 0 ? -g.sym : g.sym;
+    int cm = c;
+    if (tau) {
+        const int t1 = cl / tau, t2 = cl - t1 * tau;
+        cm = g.chan0 + t2 * tau + t1;
+    }
+    const float rm = (on && stds && tau) ? fmaxf(eps, stds[g.cumT + cm]) : 1.f;
     for (int ks = 0; ks < 2 * nkp; ++ks) {
         const int k = 4 * ks + kk, to = k >> 1;
         float v = 0.f;
@@ -156,6 +166,12 @@ __device__ __forceinline__ void pack_w_gen_lane(const float2* __restrict__ W, co
             const float2 w = W[g.cumW + (size_t)to * g.K + c];
             v = (k & 1) ? w.y : w.x;
             if (stds) v = v / r;
+            if (tau) {
+                const float2 wm = W[g.cumW + (size_t)to * g.K + cm];
+                float vm = (k & 1) ? wm.y : wm.x;
+                if (stds) vm = vm / rm;
+                v = g.sym < 0 ? v - vm : v + vm;
+            }
         }
         dst[(size_t)(ks >> 1) * 128 + (ks & 1)] = v;
     }

@@ -706,7 +706,10 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 }
 
 // ---- register-resident backward ------------------------------------------------------------
-struct BwdGeom { int l, l1, l2, rows, tau2; };
+struct BwdGeom {
+    int l, l1, l2, rows, tau2;
+    int nr1;      // slot 1: how many of the tau2 reduced channels this call takes (the first nr1)
+};
 
 // Item -> (window of two m, first output channel).  Windows are numbered from the middle of the m
 // axis outwards and the channel groups of one window are neighbours, so the lanes of a wave have
@@ -731,7 +734,7 @@ __device__ __forceinline__ void bwd_accum(const BwdGeom& q, const float* __restr
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = q.rows, tau2 = q.tau2;
     const int n_o = (SLOT == 1) ? rows : tau2;
-    const int n_r = (SLOT == 1) ? tau2 : rows;
+    const int n_r = (SLOT == 1) ? q.nr1 : rows;
     const int M_o = (SLOT == 1) ? M1 : M2, M_r = (SLOT == 1) ? M2 : M1;
     const int g_so = (SLOT == 1) ? tau2 * M : M;
     const int g_sr = (SLOT == 1) ? M : tau2 * M;
@@ -1053,7 +1056,7 @@ __device__ __forceinline__ void bwd_unit_loop_a(const BwdCtx& c, const BwdUnit& 
         const float* cgp;
         const float2 *g, *f2;
         bwd_stage<NT, TWO>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
-        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2, cur.tau2};
         bwd_accum<1, TI, RW, RM>(q, cgp, g, f2, c.rtid, ax, ay);
         bwd_stage_end<NT, TWO>(c, u, ti, t);
         if (cur.last_of_l2) {
@@ -1083,7 +1086,7 @@ __device__ __forceinline__ void bwd_unit_loop_b(const BwdCtx& c, const BwdUnit& 
         const float* cgp;
         const float2 *g, *f2;
         bwd_stage<kThreads, true>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
-        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2, cur.tau2};
 #define CGNET_CALL_B(TI_, RW_) bwd_accum<2, TI_, RW_>(q, cgp, g, c.f1, c.rtid, ax, ay)
         CGNET_BWD_SWITCH(cur.TI, cur.RW, CGNET_CALL_B)
 #undef CGNET_CALL_B
@@ -1187,7 +1190,8 @@ __device__ __forceinline__ int small_mod(int x, int n, float inv) {
 // All addresses are explicit LDS byte addresses advanced by constants from one m to the next.  The table holds zeros
 // where m - m2 is no valid m1 (every table this library fills does), so only the columns past the end of the m2
 // axis are masked; the fragment column of such an entry is clamped into its row and multiplied by that zero.
-template <int NK, bool KFULL>
+// C0: the reduction skips its first C0 steps (rows below 4 * C0 belong to somebody else: diagonal triples, below).
+template <int NK, bool KFULL, int C0 = 0>
 __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __restrict__ cgp,
                                             const float2* __restrict__ g, const float2* __restrict__ f1, int part,
                                             int split, float inv_split, int lane, f32x4 (&dre)[kHybMaxTiles],
@@ -1233,14 +1237,14 @@ __device__ __forceinline__ void bwd_mm_task(const BwdGeom& q, const float* __res
             const int fcol = max(0, min(M1 - 1, fc));             // clamped where the coefficient is zero anyway
             fc += split;
 #pragma unroll
-            for (int c = 0; c < NK; ++c) {
+            for (int c = C0; c < NK; ++c) {
                 gq[c] = lds_c(ga[c], 0);
                 ga[c] += gstep;
                 fq[c] = lds_c(fbase[c] + 8u * (unsigned)fcol, 0);
             }
             const float cv = colok ? cc : 0.f;
 #pragma unroll
-            for (int c = 0; c < NK; ++c) {
+            for (int c = C0; c < NK; ++c) {
                 const float w = KFULL ? cv : cv * kmask[c];
                 const float bx = w * fq[c].x, by = -w * fq[c].y;  // C conj(f)
                 const float ngy = -gq[c].y;
@@ -1283,7 +1287,7 @@ __device__ __forceinline__ void bwd_hybrid_loop_b(const BwdCtx& c, const BwdUnit
         const float* cgp;
         const float2 *g, *f2;
         bwd_stage<kHybThreads, false>(c, u, ti, t, cur, par, f2par, cgp, g, f2);
-        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2};
+        const BwdGeom q{cur.l, u.l1, cur.l2, u.rows, cur.tau2, cur.tau2};
         bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, lane, dre, dim);
         bwd_stage_end<kHybThreads, false>(c, u, ti, t);
         if (cur.last_of_l2) {
@@ -1407,6 +1411,7 @@ __device__ __forceinline__ int ft_l2(const FusedTask& t) { return (t.geom >> 8) 
 __device__ __forceinline__ int ft_tau2(const FusedTask& t) { return (t.geom >> 16) & 255; }
 __device__ __forceinline__ bool ft_first(const FusedTask& t) { return (t.geom >> 24) & 1; }
 __device__ __forceinline__ bool ft_last(const FusedTask& t) { return (t.geom >> 25) & 1; }
+__device__ __forceinline__ int ft_c0(const FusedTask& t) { return (t.geom >> 26) & 3; }   // diagonal triple: matrix waves skip this many steps
 __device__ __forceinline__ int ft_nks(const FusedTask& t) { return t.shape & 255; }
 __device__ __forceinline__ int ft_nch(const FusedTask& t) { return t.shape >> 16; }
 
@@ -1486,11 +1491,20 @@ __device__ __forceinline__ void gen_phase(const FusedTask& t, const float* __res
 
 // The loop over a unit's tasks, common to both roles; `work(task, table, l2 slab)` is phase 2.
 //   carried: cur = task k, nxt = task k+1 (both in scalar registers), loaded one stage before they are needed
-template <typename Work>
-__device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTask* __restrict__ ft, int ntask, Work work) {
-    FusedTask cur = ft[0];
-    FusedTask nxt = ft[min(1, ntask - 1)];
-    for (int k = 0; k < ntask; ++k) {
+//   `diag` selects the stages the call runs: false = the leading ones of ordinary triples, true = the trailing ones
+//   of diagonal triples (ft_c0 != 0; they form the last run of a unit).  A role that treats the two kinds with
+//   different code calls the loop twice, so that each loop holds a single path (a branch inside the loop that
+//   joins two matrix-core paths makes the compiler copy the accumulators at every stage).
+struct FusedCursor { FusedTask cur, nxt; int k; };
+__device__ __forceinline__ FusedCursor fused_cursor(const FusedTask* __restrict__ ft, int ntask) {
+    return FusedCursor{ft[0], ft[min(1, ntask - 1)], 0};
+}
+template <bool SPLIT, typename Work>
+__device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTask* __restrict__ ft, int ntask,
+                                                FusedCursor& cs, bool diag, Work work) {
+    for (; cs.k < ntask && (!SPLIT || (ft_c0(cs.cur) != 0) == diag); ++cs.k) {
+        const int k = cs.k;
+        const FusedTask cur = cs.cur, nxt = cs.nxt;
         dma_wait();
         __syncthreads();       // the tile's operands have landed; nobody uses the tile, the table or the l2 slab
         const FusedTask nxt2 = ft[min(k + 2, ntask - 1)];        // needed at the next stage
@@ -1507,8 +1521,8 @@ __device__ __forceinline__ void fused_task_loop(const FusedCtx& c, const FusedTa
             dma16<kHybThreads>(c.Bg + nxt.boff, c.bl, nxt.chunks >> 16, c.tid);
         }
         work(cur, reinterpret_cast<const float*>(c.cg), reinterpret_cast<const float2*>(c.f2));
-        cur = nxt;
-        nxt = nxt2;
+        cs.cur = nxt;
+        cs.nxt = nxt2;
     }
 }
 
@@ -1522,8 +1536,12 @@ __device__ __forceinline__ void fused_loop_a(const FusedCtx& c, const BwdUnit& u
         ax[i][0] = ax[i][1] = ay[i][0] = ay[i][1] = 0.f;
         tx[i][0] = tx[i][1] = ty[i][0] = ty[i][1] = 0.f;
     }
-    fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
-        const BwdGeom q{ft_l(t), u.l1, ft_l2(t), u.rows, ft_tau2(t)};
+    FusedCursor cs = fused_cursor(ft, u.task_end - u.task_begin);
+    fused_task_loop<false>(c, ft, u.task_end - u.task_begin, cs, false, [&](const FusedTask& t, const float* cgp, const float2* f2) {
+        // a diagonal triple's tile is symmetrised (see build_fused_link): this role reduces over the first 4 c0
+        // channels only, the matrix waves over the others
+        const int c0 = ft_c0(t);
+        const BwdGeom q{ft_l(t), u.l1, ft_l2(t), u.rows, ft_tau2(t), c0 ? 4 * c0 : ft_tau2(t)};
         bwd_accum<1, TI, RW, RM>(q, cgp, reinterpret_cast<const float2*>(c.tile), f2, c.tid, ax, ay);
         if (ft_last(t)) {
 #pragma unroll
@@ -1547,11 +1565,25 @@ __device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u
 #pragma unroll
     for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const float inv_split = 1.0f / (float)split;
-    fused_task_loop(c, ft, u.task_end - u.task_begin, [&](const FusedTask& t, const float* cgp, const float2* f2) {
+    const int ntask = u.task_end - u.task_begin;
+    FusedCursor cs = fused_cursor(ft, ntask);
+    // ordinary triples: the reduction over all rows; then the diagonal ones, whose first NK / 2 steps the vector
+    // waves take (build_fused_link)
+    fused_task_loop<true>(c, ft, ntask, cs, false, [&](const FusedTask& t, const float* cgp, const float2* f2) {
         const int l2 = ft_l2(t), tau2 = ft_tau2(t);
-        const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2};
-        const float2* g = reinterpret_cast<const float2*>(c.tile);
-        bwd_mm_task<NK, KFULL>(q, cgp, g, c.f1, part, split, inv_split, c.lane, dre, dim);
+        const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2, tau2};
+        bwd_mm_task<NK, KFULL, 0>(q, cgp, reinterpret_cast<const float2*>(c.tile), c.f1, part, split, inv_split, c.lane, dre, dim);
+        if (ft_last(t)) {
+            const int M2 = 2 * l2 + 1;
+            bwd_mm_store(dre, dim, tau2, M2, c.lane, part2_b + t.p2off + (size_t)part * tau2 * M2);
+#pragma unroll
+            for (int j = 0; j < kHybMaxTiles; ++j) dre[j] = dim[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+    });
+    fused_task_loop<true>(c, ft, ntask, cs, true, [&](const FusedTask& t, const float* cgp, const float2* f2) {
+        const int l2 = ft_l2(t), tau2 = ft_tau2(t);
+        const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2, tau2};
+        bwd_mm_task<NK, KFULL, NK / 2>(q, cgp, reinterpret_cast<const float2*>(c.tile), c.f1, part, split, inv_split, c.lane, dre, dim);
         if (ft_last(t)) {
             const int M2 = 2 * l2 + 1;
             bwd_mm_store(dre, dim, tau2, M2, c.lane, part2_b + t.p2off + (size_t)part * tau2 * M2);
@@ -2572,6 +2604,8 @@ int build_fused_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FusedLink*
         bop += nct * nks * 64;
         bcap = std::max(bcap, nct * nks * 256);
     }
+    bool fold = true;        // CGNET_DIAG_FOLD=0: diagonal triples take both slots like all others
+    if (const char* e = getenv("CGNET_DIAG_FOLD"); e && e[0] == '0') fold = false;
     std::vector<GenTask> gens(p->bwd_utasks.size());
     std::vector<FusedTask> ft(p->bwd_utasks.size());
     std::vector<int> map;
@@ -2591,11 +2625,21 @@ int build_fused_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FusedLink*
             g.cumW = d.cumW;
             g.K = d.K;
             g.cumT = d.cumT;
+            // Diagonal triple (l1 == l2) whose unit holds all rows: the tile g[t1][t2] and its mirror g[t2][t1] feed the
+            // same gradient, slot2(g) = slot1((-1)^l g^T) (the table is (-1)^l-symmetric under m1 <-> m2), so the
+            // weights are packed symmetrised, W'[to][(t1,t2)] = W[to][(t1,t2)]/div + (-1)^l W[to][(t2,t1)]/div', the tile
+            // made from them is g + (-1)^l g^T, and one slot's worth of arithmetic on it gives both slots' sum: the
+            // vector waves reduce over the first 4 c0 channels (slot-1 form), the matrix waves over the others (slot-2
+            // form), instead of each over all.
+            const int nk = (u.rows + 3) / 4;
+            const bool diag = fold && t.l2 == u.l1 && u.rows == p->t_F[u.l1] && nk >= 2;   // the same for a whole run of equal l2
+            const int c0 = diag ? nk / 2 : 0;
+            g.sym = diag ? ((t.l & 1) ? -u.rows : u.rows) : 0;
             gens[k] = g;
             const int nrt = (g.nch + 15) / 16;
             for (int rt = 0; rt < nrt && g.nks > 0; ++rt) { map.push_back(k); map.push_back(rt); }
             FusedTask f{};
-            f.geom = t.l | (t.l2 << 8) | (t.tau2 << 16) | (t.first_of_l2 << 24) | (t.last_of_l2 << 25);
+            f.geom = t.l | (t.l2 << 8) | (t.tau2 << 16) | (t.first_of_l2 << 24) | (t.last_of_l2 << 25) | (c0 << 26);
             f.offF2p = t.offF2p;
             f.cgp_off = t.cgp_off;
             f.cgp_len = t.cgp_len;

@@ -585,11 +585,15 @@ def _fused_backward_cases(n, seed):
                     (20, [16] * 21, [16] * 21, 1, False, True, n + 2)]
 
 
+@pytest.mark.parametrize("fold", [False, True])
 @pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _fused_backward_cases(12, 31))
-def test_fused_backward_equals_two_kernel_backward(dev, lmax, tin, tout, bsz, sparse, bn, k):
-    """The one-kernel backward (gFF tiles formed in LDS) returns bit for bit what the gFF kernel followed by the
-    product's backward returns, for the input gradient and the weight gradient, in training mode; the small
-    cases are also held against the oracle."""
+def test_fused_backward_equals_two_kernel_backward(dev, monkeypatch, lmax, tin, tout, bsz, sparse, bn, k, fold):
+    """The one-kernel backward (gFF tiles formed in LDS) against the gFF kernel followed by the product's backward, for the
+    input gradient and the weight gradient, in training mode.  Without the fold of the diagonal triples
+    (CGNET_DIAG_FOLD=0 when the layer plan is made) the two routes agree bit for bit; with it (the default) the triples
+    with l1 = l2 are summed in another order (symmetrised tile, one slot's arithmetic), so the input gradients agree to
+    rounding.  The small cases are also held against the oracle."""
+    monkeypatch.setenv("CGNET_DIAG_FOLD", "1" if fold else "0")
     mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=400 + k)
     lp = mod.native_layer_plan()
     if not lp.fused_backward_supported:
@@ -609,7 +613,13 @@ def test_fused_backward_equals_two_kernel_backward(dev, lmax, tin, tout, bsz, sp
         x = x64.float().to(dev).requires_grad_(True)
         mod(x, straight_output=True).backward(go)
         grads.append((x.grad.clone(), mod.bnWMM.W.grad.clone() if mod.bnWMM.W.numel() else None))
-    assert torch.equal(grads[0][0], grads[1][0]), "input gradient differs: max %.3e" % float((grads[0][0] - grads[1][0]).abs().max())
+    if fold:
+        # per degree: the difference is rounding of sums of that degree's magnitude
+        scale = float(grads[0][0].abs().max())
+        err = float((grads[0][0] - grads[1][0]).abs().max())
+        assert err <= 2e-5 * scale + 1e-30, "input gradient differs: max %.3e at scale %.3e" % (err, scale)
+    else:
+        assert torch.equal(grads[0][0], grads[1][0]), "input gradient differs: max %.3e" % float((grads[0][0] - grads[1][0]).abs().max())
     if grads[0][1] is not None:
         assert torch.equal(grads[0][1], grads[1][1])
     if lmax <= 8:
