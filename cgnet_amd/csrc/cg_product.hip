@@ -706,6 +706,11 @@ cg_backward_kernel(const float2* __restrict__ F, const float2* __restrict__ gFF,
 }
 
 // ---- register-resident backward ------------------------------------------------------------
+// diagonal triples in the fused layer backward: of the NK reduction steps of four rows the vector waves take the
+// first CGNET_DIAG_C0(NK), the matrix waves the others (rounding up instead of down measured the same)
+#ifndef CGNET_DIAG_C0
+#define CGNET_DIAG_C0(NK_) ((NK_) / 2)
+#endif
 struct BwdGeom {
     int l, l1, l2, rows, tau2;
     int nr1;      // slot 1: how many of the tau2 reduced channels this call takes (the first nr1)
@@ -1583,7 +1588,7 @@ __device__ __forceinline__ void fused_loop_b(const FusedCtx& c, const BwdUnit& u
     fused_task_loop<true>(c, ft, ntask, cs, true, [&](const FusedTask& t, const float* cgp, const float2* f2) {
         const int l2 = ft_l2(t), tau2 = ft_tau2(t);
         const BwdGeom q{ft_l(t), u.l1, l2, u.rows, tau2, tau2};
-        bwd_mm_task<NK, KFULL, NK / 2>(q, cgp, reinterpret_cast<const float2*>(c.tile), c.f1, part, split, inv_split, c.lane, dre, dim);
+        bwd_mm_task<NK, KFULL, CGNET_DIAG_C0(NK)>(q, cgp, reinterpret_cast<const float2*>(c.tile), c.f1, part, split, inv_split, c.lane, dre, dim);
         if (ft_last(t)) {
             const int M2 = 2 * l2 + 1;
             bwd_mm_store(dre, dim, tau2, M2, c.lane, part2_b + t.p2off + (size_t)part * tau2 * M2);
@@ -2633,7 +2638,7 @@ int build_fused_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FusedLink*
             // form), instead of each over all.
             const int nk = (u.rows + 3) / 4;
             const bool diag = fold && t.l2 == u.l1 && u.rows == p->t_F[u.l1] && nk >= 2;   // the same for a whole run of equal l2
-            const int c0 = diag ? nk / 2 : 0;
+            const int c0 = diag ? CGNET_DIAG_C0(nk) : 0;
             g.sym = diag ? ((t.l & 1) ? -u.rows : u.rows) : 0;
             gens[k] = g;
             const int nrt = (g.nch + 15) / 16;

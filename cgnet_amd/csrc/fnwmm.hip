@@ -26,7 +26,8 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kStatTileBytes = 32 * 1024;
 constexpr int kStatGroups = 8;
-constexpr int kGradWChunk = 32;     // samples whose weight-gradient sums one work-group forms
+constexpr int kGradWChunk = 32;     // samples whose weight-gradient sums one work-group forms, at most (the chunks of a
+                                    // batch are made equal: 100 samples are four chunks of 25, not 32 + 32 + 32 + 4)
 constexpr int kGradWFold = 4;       // samples per matrix-core chain inside a chunk
 
 // --------------------------------------------------------------------------- statistics
@@ -1047,11 +1048,13 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_HIP(hipGetLastError());
         } else {
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
-            const int nchunks = gradw_chunks(B);
+            // equal chunks of at most kGradWChunk samples; the kernel derives the number of chunks from their size
+            const int spc = (B + gradw_chunks(B) - 1) / gradw_chunks(B);
+            const int nchunks = (B + spc - 1) / spc;             // <= gradw_chunks(B), what the workspace holds
             const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
             CGNET_LAUNCH(wmm_gradw_kernel, dim3(grid_1d(plan->gw_units.size(), nchunks)), dim3(kThreads), lds, s,
                                (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
-                               kGradWChunk, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
+                               spc, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
             CGNET_HIP(hipGetLastError());
             CGNET_LAUNCH(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)gw_part, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg,
