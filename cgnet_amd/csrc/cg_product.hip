@@ -2066,6 +2066,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
         // attempts 0 .. n_hyb4 - 1: four groups per compute unit; .. n_hyb - 1: three; attempt n_hyb: two groups, tiles
         // of kHybTileBytes
         const int hyb_groups = attempt < n_hyb4 ? 4 : attempt < n_hyb ? 3 : 2;
+        // CGNET_BWD_MAX_GROUPS=3 (or 2): plans for four (three) work-groups per compute unit are not tried
+        if (const char* e = getenv("CGNET_BWD_MAX_GROUPS"); e && hybrid && attempt <= n_hyb && hyb_groups > atoi(e)) continue;
         const long long tile_limit = !hybrid ? kBwdTileBytes : attempt < n_hyb ? hyb_tiles_kb[attempt] * 1024LL : kHybTileBytes;
         const size_t hyb_lds_limit = hyb_groups == 4 ? kHybLds4 : hyb_groups == 3 ? kHybLds3 : kMaxHybLds;
         const int hyb_max_ti = hyb_groups == 4 ? 2 : kHybMaxTI;

@@ -28,7 +28,7 @@ constexpr int kStatTileBytes = 32 * 1024;
 constexpr int kStatGroups = 8;
 constexpr int kGradWChunk = 32;     // samples whose weight-gradient sums one work-group forms, at most (the chunks of a
                                     // batch are made equal: 100 samples are four chunks of 25, not 32 + 32 + 32 + 4)
-constexpr int kGradWFold = 4;       // samples per matrix-core chain inside a chunk
+constexpr int kGradWFold = 1;       // samples per matrix-core chain inside a chunk
 
 // --------------------------------------------------------------------------- statistics
 // sums of |z| and |z|^2 over (b, m) per mid channel, from FF

@@ -6,13 +6,18 @@ cannot hold that bar on sums whose terms are much larger than the result (weight
 normalised by a small running std reach 1e2; an entry that cancels to ~0 still carries the rounding of
 its large terms).  How much of that is the arithmetic's and how much the GPU's is measured, not assumed: every
 comparison also evaluates the oracle in float32 on the CPU (the reference's own precision), and the GPU
-must satisfy
+must satisfy, with E = max|cpu32 - oracle64| over the tensor,
 
-    |gpu - oracle64|  <=  max( 1e-6 + 1e-5 * |oracle64| ,  4 * max|cpu32 - oracle64| )      elementwise,
+    |gpu - oracle64|  <=  max( 1e-6 + 1e-5 * |oracle64| ,  3 E )      elementwise, except that
+    at most one element in 5000 may lie between 3 E and 4 E, and none beyond 4 E;
+    rms(gpu - oracle64) <= 3 rms(cpu32 - oracle64) + 1e-7 rms(oracle64)   for tensors of 64 elements or more,
 
-i.e. it is held to the strict bar wherever the float32 CPU path itself meets it, and otherwise to four times that
+i.e. it is held to the strict bar wherever the float32 CPU path itself meets it, and otherwise to three times that
 path's worst error on the same tensor (the CPU path sums through BLAS in blocks, the kernels in chains of up to a
-few hundred terms, so worst-case errors two to three times the CPU's are the order of summation, not a defect).  Both maxima are printed (``pytest -s``) and, when the
+few hundred terms, so worst-case errors two to three times the CPU's are the order of summation, not a defect; the
+root-mean-square errors, a steadier measure than maxima, differ by a factor 1.0 in the median over the suite).  The
+tail allowance covers entries that are zero by symmetry and consist of rounding noise divided by max(eps, std) =
+1e-5 (one such element of 116 million lies at 3.2 E).  Both maxima are printed (``pytest -s``) and, when the
 environment variable CGNET_PARITY_REPORT names a file, appended to it as JSON lines.
 """
 import json
@@ -30,7 +35,8 @@ from oracle import triples as OT
 pytestmark = pytest.mark.gpu
 
 RTOL, ATOL = 1e-5, 1e-6
-TWIN_FACTOR = 4.0
+TWIN_FACTOR, TWIN_TAIL_FACTOR, TWIN_TAIL_SHARE = 3.0, 4.0, 1.0 / 5000
+RMS_FACTOR = 3.0
 F64, F32 = torch.float64, torch.float32
 
 
@@ -58,6 +64,7 @@ def assert_close(got, ref, what, twin=None, rtol=RTOL, atol=ATOL):
     err = (got - ref).abs()
     err_twin = float((_flat(twin) - ref).abs().max()) if twin is not None else 0.0
     bound = torch.clamp(strict, min=TWIN_FACTOR * err_twin)
+    outer = torch.clamp(strict, min=TWIN_TAIL_FACTOR * err_twin)
     rms = lambda e: float(torch.sqrt(torch.mean(e * e)))
     rec = {"test": os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0], "what": what, "n": ref.numel(),
            "max_ref": float(ref.abs().max()), "err_gpu": float(err.max()), "err_cpu32": err_twin if twin is not None else None,
@@ -72,10 +79,13 @@ def assert_close(got, ref, what, twin=None, rtol=RTOL, atol=ATOL):
         with open(path, "a") as fh:
             fh.write(json.dumps(rec) + "\n")
     worst = int(torch.argmax(err - bound))
-    assert bool((err <= bound).all()), (
+    n_tail = int((err > bound).sum())
+    assert n_tail <= math.ceil(TWIN_TAIL_SHARE * ref.numel()) and bool((err <= outer).all()), (
         "%s: %d of %d outside tolerance; worst |err|=%.3e at %d (ref %.6e, bound %.3e, cpu32 max err %.3e)"
-        % (what, int((err > bound).sum()), ref.numel(), float(err[worst]), worst, float(ref[worst]),
-           float(bound[worst]), err_twin))
+        % (what, n_tail, ref.numel(), float(err[worst]), worst, float(ref[worst]), float(bound[worst]), err_twin))
+    if twin is not None and ref.numel() >= 64 and rec["strict_violations_gpu"] > 0:
+        assert rec["rms_gpu"] <= RMS_FACTOR * rec["rms_cpu32"] + 1e-7 * rms(ref), (
+            "%s: rms error %.3e against %.3e of the float32 CPU path" % (what, rec["rms_gpu"], rec["rms_cpu32"]))
 
 
 def make_codes(lmax, mode):
@@ -853,6 +863,43 @@ def test_full_size_layer_config3_runs(dev):
     out2 = mod2(x.detach(), straight_output=True)
     assert torch.allclose(out, out2, rtol=1e-5, atol=1e-6)
     assert torch.allclose(mod.bnWMM.bn_stds, mod2.bnWMM.bn_stds, rtol=1e-6, atol=1e-9)
+
+
+@pytest.mark.timeout(600)
+def test_full_size_layer_config3_against_oracle(dev):
+    """Benchmark configuration 3 at its own batch (L=11, tau=12, B=100), held against the oracle rather than against
+    itself.  With fixed statistics (evaluation mode) the layer acts on every sample alone and its weight gradient is the
+    sum of the samples' weight gradients: the output and the input gradient of three samples of the batch (the first,
+    one inside, the last: a full chunk and the partial last one of every kernel) and the weight gradient of the whole
+    batch (the oracle evaluated in chunks of 25 samples and added up) are compared, on both backward routes."""
+    lmax, tau, bsz = 11, [12] * 12, 100
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tau, tau, False, True, seed=3)
+    mod.eval()
+    ora.training = twin.training = False
+    x64 = rand_straight(tau, bsz, seed=33)
+    go64 = randn32((bsz, 1728, 2), torch.Generator().manual_seed(35))
+    # the oracle: per chunk of samples, float64 and float32
+    outs, gxs, gw, tw_outs, tw_gxs, tw_gw = [], [], 0, [], [], 0
+    for b0 in range(0, bsz, 25):
+        sl = slice(b0, b0 + 25)
+        o, gx, g = oracle_step(ora, x64[sl], w64, go64[sl])
+        outs.append(o); gxs.append(gx); gw = gw + g
+        o, gx, g = oracle_step(twin, x64[sl], w64, go64[sl], dtype=F32)
+        tw_outs.append(o); tw_gxs.append(gx); tw_gw = tw_gw + g.double()
+    want, want_gx = torch.cat(outs), torch.cat(gxs)
+    tw, tw_gx = torch.cat(tw_outs), torch.cat(tw_gxs)
+    pick = [0, 57, 99]
+    for fused_backward in (True, False):
+        mod.fused_backward = fused_backward
+        mod.bnWMM.W.grad = None
+        x = x64.float().to(dev).requires_grad_(True)
+        out = mod(x, straight_output=True)
+        out.backward(go64.float().to(dev))
+        tag = " (one-kernel backward)" if fused_backward else " (two-kernel backward)"
+        assert_close(out[pick], want[pick], "config 3, B=100: forward of three samples" + tag, tw[pick])
+        assert_close(x.grad[pick], want_gx[pick], "config 3, B=100: grad F of three samples" + tag, tw_gx[pick])
+        assert_close(mod.bnWMM.W.grad, gw, "config 3, B=100: grad W of the batch" + tag, tw_gw)
+    assert mod.bnWMM.bn_cnt == 1.0
 
 
 @pytest.mark.parametrize("sparse", [True, False])
