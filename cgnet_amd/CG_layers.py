@@ -141,13 +141,18 @@ class MyBatchNormWeightMM_cuda(nn.Module):
             self.bn_cnt += 1
         return output
 
-    # ``bn_cnt`` stays the plain float attribute of the reference (CG_layers.py:92,130: read on every forward, so
-    # it must not live on the device), but unlike there it travels with ``state_dict`` as the entry ``bn_cnt``,
-    # so a resumed run continues the moving average where it stopped.  Checkpoints written by the reference lack
-    # the entry: loading them keeps the current count.
+    # ``bn_cnt`` is the plain float attribute of the reference (CG_layers.py:92,130: read on every forward, so it
+    # must not live on the device) and, as there, is NOT part of ``state_dict`` by default: the key set is exactly the
+    # reference's (``W``, ``bn_stds``, ``bn_eps``), so checkpoints load with ``strict=True`` in both directions.  The
+    # reference loses the count on a resume; ``persist_bn_cnt = True`` (on the class or on an instance) adds the entry
+    # ``bn_cnt`` to ``state_dict`` so that a resumed run continues the moving average where it stopped -- such a
+    # checkpoint is rejected by the reference's strict loader.  A ``bn_cnt`` entry is accepted on load either way.
+    persist_bn_cnt = False
+
     def _save_to_state_dict(self, destination, prefix, keep_vars):
         super()._save_to_state_dict(destination, prefix, keep_vars)
-        destination[prefix + "bn_cnt"] = torch.tensor(float(self.bn_cnt), dtype=torch.float64)
+        if self.persist_bn_cnt:
+            destination[prefix + "bn_cnt"] = torch.tensor(float(self.bn_cnt), dtype=torch.float64)
 
     def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
                               error_msgs):

@@ -99,7 +99,7 @@ struct cgnet_cg_plan {
     cgnet::BwdUnit* d_bwd_units = nullptr;
     cgnet::BwdUTask* d_bwd_utasks = nullptr;
     int* d_bwd_combine = nullptr;                // [L+2] cumF | [L+1] own1 | [L+2] list begin | list of slab offsets
-    int* d_bwd_padmeta = nullptr;                // [L+2] cumF | [L+2] cumFp | per triple {cg_off, cgp_off, cgp_len, M, M2}
+    int* d_bwd_padmeta = nullptr;                // [L+2] cumF | [L+2] cumFp | per triple {cg_off, cgp_off, cgp_len, M, M2, l1}
     int bwd_nFp = 0;                             // complex entries of one sample's padded fragments
     int bwd_cgp_len = 0;                         // floats of all padded tables
     int bwd_f1cap = 0, bwd_f2cap = 0, bwd_cgcap = 0, bwd_tcap = 0;   // LDS bytes of the staged operands
@@ -195,13 +195,24 @@ __device__ __forceinline__ void pad_fragments_block(const float2* __restrict__ F
     Fp[idx] = v;
 }
 
-// One triple's table between kTabLo / kTabHi zero rows, by one work-group.  m: {cg_off, cgp_off, cgp_len, M, M2}
+// One triple's table between kTabLo / kTabHi zero rows, by one work-group.  m: {cg_off, cgp_off, cgp_len, M, M2, l1}.
+// Entries whose m1 = m - m2 is no valid index of degree l1 become zeros whatever the caller's table holds there: the
+// matrix-core half of the backward multiplies them with neighbouring fragment entries and relies on the product
+// being zero.
+constexpr int kPadMetaInts = 6;
 __device__ __forceinline__ void pad_table_block(const float* __restrict__ CG, float* __restrict__ CGP,
                                                 const int* __restrict__ m) {
-    const int cg_off = m[0], cgp_off = m[1], len = m[2], M = m[3], M2 = m[4];
+    const int cg_off = m[0], cgp_off = m[1], len = m[2], M = m[3], M2 = m[4], l1 = m[5];
+    const int l = (M - 1) >> 1, l2 = (M2 - 1) >> 1;
     for (int e = threadIdx.x; e < len; e += blockDim.x) {
         const int x = e - kTabLo * M2;
-        CGP[cgp_off + e] = (x >= 0 && x < M * M2) ? CG[cg_off + x] : 0.f;
+        float v = 0.f;
+        if (x >= 0 && x < M * M2) {
+            const int r = x / M2, c = x - r * M2;
+            const int m1 = (r - l) - (c - l2);
+            if (m1 >= -l1 && m1 <= l1) v = CG[cg_off + x];
+        }
+        CGP[cgp_off + e] = v;
     }
 }
 

@@ -413,10 +413,13 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
     const int b0 = group * samples_per_group;
     const int b1 = min(B, b0 + samples_per_group);
     if (b0 < b1) issue(b0, 0);
-    // the table with three zeros behind every row (the zeros are the cleared LDS)
+    // the table with three zeros behind every row (the zeros are the cleared LDS); entries whose m1 = m - m2 is no
+    // valid index of degree l1 are staged as zeros whatever the caller's table holds there (the kernel multiplies
+    // them with neighbouring fragment entries and relies on the product being zero)
     for (int e = tid; e < M * M2; e += kFwdMmThreads) {
-        const int r = e / M2;
-        cg[r * P + (e - r * M2)] = CG[t.cg_off + e];
+        const int r = e / M2, c = e - r * M2;
+        const int m1 = (r - t.l) - (c - t.l2);
+        cg[r * P + c] = (m1 >= -t.l1 && m1 <= t.l1) ? CG[t.cg_off + e] : 0.f;
     }
     int par = 0;
     for (int b = b0; b < b1; ++b, par ^= 1) {
@@ -1688,7 +1691,7 @@ cg_backward_pad_kernel(const float2* __restrict__ F, const float* __restrict__ C
                        int nbF) {
     __shared__ int s_tab[kMaxLookup];
     if ((int)blockIdx.x < nbF) pad_fragments_block(F, Fp, meta, L, nF, nFp, B, (int)blockIdx.x, s_tab);
-    else pad_table_block(CG, CGP, meta + 2 * (L + 2) + 5 * ((int)blockIdx.x - nbF));
+    else pad_table_block(CG, CGP, meta + 2 * (L + 2) + kPadMetaInts * ((int)blockIdx.x - nbF));
 }
 
 // gF[b][e] = slot-1 part (if any unit owns the degree) + the slot-2 slabs of that degree, in list order
@@ -2274,8 +2277,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
             pad_meta.insert(pad_meta.end(), p->cumF.begin(), p->cumF.end());           // L+2
             pad_meta.insert(pad_meta.end(), cumFp.begin(), cumFp.end());               // L+2
             for (int i = 0; i < nllls; ++i) {
-                const int v[5] = {cgo[i], cgp_off[i], cgp_off[i + 1] - cgp_off[i], 2 * tl[i] + 1, 2 * tl2[i] + 1};
-                pad_meta.insert(pad_meta.end(), v, v + 5);
+                const int v[kPadMetaInts] = {cgo[i], cgp_off[i], cgp_off[i + 1] - cgp_off[i], 2 * tl[i] + 1, 2 * tl2[i] + 1, tl1[i]};
+                pad_meta.insert(pad_meta.end(), v, v + kPadMetaInts);
             }
             if (const char* dbg = getenv("CGNET_DEBUG"); dbg && dbg[0] == '1') {
                 fprintf(stderr, "[cgnet] backward units=%zu tasks=%zu P2=%d lds=%zu%s\n", p->bwd_units.size(),
@@ -2302,7 +2305,8 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
 
     CGNET_HIP(hipGetDevice(&p->device));
     // set-up time: the statistics area of cgnet_sparse_forward_stats_static gets its address on this device
-    CGNET_REQUIRE(resolve_static_scratch() != nullptr, CGNET_ERR_HIP, "%s", cgnet_last_error());
+    // (a plan is usable without it: a failure here is reported by that entry point, which resolves the address again)
+    if (!resolve_static_scratch()) clear_error();
     if (!p->fwd_tasks.empty()) {
         CGNET_HIP(hipMalloc((void**)&p->d_fwd_tasks, sizeof(CgTask) * p->fwd_tasks.size()));
         CGNET_HIP(hipMemcpy(p->d_fwd_tasks, p->fwd_tasks.data(), sizeof(CgTask) * p->fwd_tasks.size(), hipMemcpyHostToDevice));
@@ -2469,7 +2473,7 @@ extern "C" int cgnet_sparse_forward_stats_static(const cgnet_cg_plan* plan, cons
                   "the partial statistics of this call need %zu bytes, the static area holds %zu "
                   "(use cgnet_sparse_forward_stats with a caller workspace)", need, kStaticScratchBytes);
     void* area = resolve_static_scratch();   // resolved when the plan was created on this device; a lookup here
-    CGNET_REQUIRE(area, CGNET_ERR_HIP, "%s", cgnet_last_error());
+    if (!area) return CGNET_ERR_HIP;         // resolve_static_scratch has recorded the message
     const int spg = samples_per_group_for(B, (int)plan->fwd_tasks.size());
     const int ngroups = (B + spg - 1) / spg;
     // every partial sum [group][channel][2] of this call is written by the product kernel before the

@@ -76,7 +76,7 @@ layer_prepare_kernel(const float2* __restrict__ W, const float* __restrict__ std
         return;
     }
     blk -= nbF;
-    pad_table_block(CG, CGP, padmeta + 2 * (L + 2) + 5 * blk);
+    pad_table_block(CG, CGP, padmeta + 2 * (L + 2) + kPadMetaInts * blk);
 }
 
 struct SavedAreas { size_t Ag, Fp, CGP, total; };

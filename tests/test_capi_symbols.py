@@ -77,8 +77,23 @@ def test_modules_hold_reference_parameter_layout_without_a_gpu():
     net = CGNet.SphericalCNN(lmax, [[1] * (lmax + 1)] + [taus] * 5, device="cpu")
     shapes = [tuple(p.shape) for p in net.parameters() if p.requires_grad]
     assert shapes == [(1643, 2)] + [(31023, 2)] * 4          # MNIST/example.sh:12 of the reference
-    keys = list(net.state_dict().keys())
-    assert "cgs.0.bnWMM.W" in keys and "cgs.0.bnWMM.bn_stds" in keys and "cgs.0.bnWMM.bn_eps" in keys
+    # the state dictionary holds exactly the reference's entries (CGNet/CG_layers.py:89-91,116-122: three Parameters per
+    # layer, nothing else), so checkpoints pass the reference's strict load_state_dict in both directions
+    want = {"cgs.%d.bnWMM.%s" % (i, k) for i in range(5) for k in ("W", "bn_stds", "bn_eps")}
+    assert set(net.state_dict().keys()) == want
+    # opt-in: the moving-average count as a fourth entry (the reference loses it on a resume)
+    from cgnet_amd import CG_layers
+    net.cgs[2].bnWMM.persist_bn_cnt = True
+    net.cgs[2].bnWMM.bn_cnt = 5.0
+    sd = net.state_dict()
+    assert set(sd.keys()) == want | {"cgs.2.bnWMM.bn_cnt"} and float(sd["cgs.2.bnWMM.bn_cnt"]) == 5.0
+    net.cgs[2].bnWMM.bn_cnt = 1.0
+    net.load_state_dict(sd)                                   # strict: the extra entry is consumed, not "unexpected"
+    assert net.cgs[2].bnWMM.bn_cnt == 5.0
+    net.cgs[2].bnWMM.persist_bn_cnt = False
+    assert not CG_layers.MyBatchNormWeightMM_cuda.persist_bn_cnt
+    net.load_state_dict({k: v for k, v in sd.items() if not k.endswith("bn_cnt")})   # a reference checkpoint
+    assert net.cgs[2].bnWMM.bn_cnt == 5.0                     # ... leaves the count alone
     assert net.output_length == 122
     import torch
     with pytest.raises(AssertionError):

@@ -641,6 +641,51 @@ def test_fused_backward_equals_two_kernel_backward(dev, monkeypatch, lmax, tin, 
         check_layer_step(dev, mod, ora, twin, w64, x64, go.double().cpu())
 
 
+def test_invalid_table_slots_are_never_used(dev):
+    """Slots of the flat table whose m1 = m - m2 is no index of degree l1 carry no coefficient; the reference's
+    kernels never read them (cudaCG_sparse.cu:164,243).  Here the matrix-core kernels walk over them, so every
+    staged copy of the table masks them: NaNs in those slots change no result, bit for bit (product forward and
+    backward, the layer's forward and its one-kernel backward)."""
+    from cgnet_amd import CG_layers
+    lmax, tin, tout, bsz = 5, [9, 8, 12, 10, 16, 8], [8, 3, 5, 16, 3, 7], 3
+    mod, _, _, _ = build_layer_pair(dev, lmax, tin, tout, False, True, seed=13)
+    cgmod, bn, lp = mod.cg, mod.bnWMM, mod.native_layer_plan()
+    assert lp.fused_backward_supported, lp.fused_backward_reason
+    clean = cgmod.CGspace.clone()
+    dirty = clean.clone()
+    offs = [int(v) for v in cgmod._cg_offsets_host]
+    n_bad = 0
+    for i, (l, l1, l2) in enumerate(OT.decode(lmax, cgmod.lll_list)):
+        t = dirty[offs[i]:offs[i + 1]].view(2 * l + 1, 2 * l2 + 1)
+        m = torch.arange(-l, l + 1, device=dev).view(-1, 1)
+        m2 = torch.arange(-l2, l2 + 1, device=dev).view(1, -1)
+        bad = (m - m2).abs() > l1
+        assert bool((t[bad] == 0).all())                 # the library writes zeros there
+        t[bad] = float("nan")
+        n_bad += int(bad.sum())
+    assert n_bad > 0
+    x = rand_straight(tin, bsz, seed=51).float().to(dev)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go = torch.randn(bsz, n_o, 2, generator=torch.Generator().manual_seed(53)).to(dev)
+    plan = cgmod.native_plan()
+    results = []
+    for table in (clean, dirty):
+        FF = torch.empty(bsz, plan.nFF, 2, device=dev)
+        plan.forward(x, FF, table, bsz)
+        gFF = torch.randn(bsz, plan.nFF, 2, generator=torch.Generator().manual_seed(55)).to(dev)
+        gF = torch.empty_like(x)
+        plan.backward(x, gF, gFF, table, bsz)
+        FF2, out = torch.empty_like(FF), torch.empty(bsz, n_o, 2, device=dev)
+        stds = bn.bn_stds.detach().clone()
+        saved = lp.forward(x, FF2, out, bn.W.detach(), table, bsz, stds, 1.0, bn._eps_host, 0x1 | 0x2, save=True)
+        gF2 = torch.empty_like(x)
+        lp.backward_fused(x, gF2, go, bn.W.detach(), table, bsz, stds, bn._eps_host, 0x1 | 0x2, saved)
+        results.append((FF, gF, FF2, out, stds, gF2))
+    for a, b in zip(*results):
+        assert torch.isfinite(b).all()
+        assert torch.equal(a, b)
+
+
 def _random_layer_cases(n, seed, out_lo=1):
     rng = np.random.default_rng(seed)
     cases = []
@@ -858,7 +903,7 @@ def test_full_size_layer_config3_runs(dev):
     mod2.load_state_dict(mod.state_dict())
     with torch.no_grad():
         mod2.bnWMM.bn_stds.fill_(1.0)
-    mod2.bnWMM.bn_cnt = 1.0                               # the state dictionary carried the advanced count
+    assert mod2.bnWMM.bn_cnt == 1.0                       # the count is no part of the state dictionary (as in the reference)
     mod2.fused = False
     out2 = mod2(x.detach(), straight_output=True)
     assert torch.allclose(out, out2, rtol=1e-5, atol=1e-6)
@@ -1025,14 +1070,20 @@ def test_classifier_from_coefficient_file(dev, tmp_path):
     assert counts == {"SphericalCNN.cgs.0.bnWMM": 2.0, "SphericalCNN.cgs.1.bnWMM": 2.0}
     net2 = model.MNIST_Net(n_deg - 1, tau_type=2, tau_man=4, nlayers=2, dropout=None)
     sd = net.state_dict()
-    assert float(sd["SphericalCNN.cgs.1.bnWMM.bn_cnt"]) == 2.0     # the count travels with the checkpoint
-    net2.load_state_dict(sd)
-    assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
-    # a checkpoint written by the reference has no such entry: it loads, and the helper restores the counts
+    assert not any(k.endswith("bn_cnt") for k in sd)              # the reference's key set, nothing added
+    # as with a checkpoint of the reference, the counts are not in it: it loads, and the helper restores them
     net2.SphericalCNN.cgs[1].bnWMM.bn_cnt = 7.0
-    net2.load_state_dict({k: v for k, v in sd.items() if not k.endswith("bn_cnt")})
+    net2.load_state_dict(sd)
     assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 7.0
     CGNet.load_normalisation_counts(net2, counts)
+    assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
+    # opt-in: the count travels with the checkpoint
+    for cg in net.SphericalCNN.cgs:
+        cg.bnWMM.persist_bn_cnt = True
+    sd2 = net.state_dict()
+    assert float(sd2["SphericalCNN.cgs.1.bnWMM.bn_cnt"]) == 2.0
+    net2.SphericalCNN.cgs[1].bnWMM.bn_cnt = 9.0
+    net2.load_state_dict(sd2)
     assert net2.SphericalCNN.cgs[1].bnWMM.bn_cnt == 2.0
     net.eval(); net2.eval()
     assert torch.equal(net(x), net2(x))

@@ -46,6 +46,13 @@ def test_static_area_entry_point_matches_workspace_entry_point():
         got_sums = torch.full_like(want_sums, float("nan"))
         plan.forward_stats_static(x, got_ff, cg, bsz, got_sums)
         torch.cuda.synchronize()
+        # the call allocates nothing: the device's free memory is the same before and after a second call on
+        # the same buffers (torch's caching allocator is not involved: the binding passes raw pointers only)
+        free_before, _ = torch.cuda.mem_get_info(dev)
+        plan.forward_stats_static(x, got_ff, cg, bsz, got_sums)
+        torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info(dev)
+        assert free_after == free_before, "the entry point changed the device's free memory by %d bytes" % (free_before - free_after)
         assert torch.isfinite(got_ff).all() and torch.isfinite(got_sums).all()
         assert torch.equal(got_ff, want_ff), "product differs at B=%d" % bsz
         assert torch.equal(got_sums, want_sums), "statistics differ at B=%d" % bsz
