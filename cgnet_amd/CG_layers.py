@@ -383,8 +383,13 @@ class _CGBN_fused(torch.autograd.Function):
         # the operands of the one-kernel backward are prepared beside those of the mixing forward, in the same launch
         saved_ops = layer_plan.forward(Fs, FF, out, W, CG, B, bn_stds, float(bn_cnt), float(bn_eps), flags,
                                        save=ctx.fused_backward and ctx.needs_input_grad[0])
-        # bn_stds was updated in place; backward must see the value used for this batch
-        saved_stds = bn_stds.detach().clone() if (bn_stds is not None and need_grad) else None
+        # bn_stds was updated in place; backward must see the value used for this batch: the copy the forward left
+        # among the saved operands, else a clone
+        saved_stds = None
+        if bn_stds is not None and need_grad:
+            saved_stds = layer_plan.saved_stds(saved_ops, B)
+            if saved_stds is None:
+                saved_stds = bn_stds.detach().clone()
         ctx.layer_plan, ctx.B, ctx.eps, ctx.flags = layer_plan, B, float(bn_eps), flags
         ctx.save_for_backward(Fs, W, FF, CG, saved_stds, saved_ops)
         return out

@@ -48,6 +48,7 @@ SIGNATURES = {
     "cgnet_CGBN_backward_fused_supported": (ctypes.c_int, [_vp]),
     "cgnet_CGBN_backward_fused_reason": (ctypes.c_char_p, [_vp]),
     "cgnet_CGBN_saved_bytes": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_saved_stds_bytes": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_CGBN_forward_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_CGBN_forward": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                           ctypes.c_float, ctypes.c_int, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp]),

@@ -239,7 +239,8 @@ class LayerPlan:
 
     def forward(self, F, FF, O, W, CG, B, stds, cnt, eps, flags, save=True):
         """O = layer(F); FF is written too.  Returns the saved-operand tensor for ``backward_fused`` (None when
-        ``save`` is false or the fused backward is not supported)."""
+        ``save`` is false or the fused backward is not supported); ``saved_stds`` is the view of it that holds the
+        stds this batch was normalised with."""
         cg, wmm = self.cg_plan, self.wmm_plan
         cg._check_io(F, B)
         _require_gpu("FF", FF)
@@ -266,6 +267,13 @@ class LayerPlan:
                                               0 if saved is None else saved.numel(), _ptr(ws), ws.numel(),
                                               _stream(F.device)))
         return saved
+
+    def saved_stds(self, saved, B):
+        """The float32 view of the stds copy inside a saved-operand tensor (None if it holds none)."""
+        if saved is None:
+            return None
+        n = int(_lib.load().cgnet_CGBN_saved_stds_bytes(self._h, int(B)))
+        return saved[:n].view(torch.float32) if n else None
 
     def backward_fused(self, F, gF, gO, W, CG, B, stds, eps, flags, saved=None):
         """gF of the whole layer straight from gO (no gFF in memory): cgnet_CGBN_backward_fused."""

@@ -52,12 +52,15 @@ fn_finish_kernel(const double* __restrict__ part, int ngroups, float* __restrict
 //   [.., + nb_gen)   packed weights of the fused backward, four (task, row tile) pairs each   (pack_w_gen_lane)
 //   [.., + nbF)      fragments with a zero behind every row             (pad_fragments_block)
 //   [.., + ntab)     every triple's table between zero rows             (pad_table_block)
+//   [.., + nb_std)   a copy of the stds (the running values move on with the next batch; the backward of this one
+//                    needs those it was normalised with)
 __global__ void __launch_bounds__(256)
 layer_prepare_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
                      const WmmDeg* __restrict__ degs, int ndeg, float* __restrict__ Wp, int wp_blocks, int nb_fwd,
                      const GenTask* __restrict__ gens, const int* __restrict__ packmap, int npack, float* __restrict__ Ag,
                      int nb_gen, const float2* __restrict__ F, const float* __restrict__ CG, float2* __restrict__ Fp,
-                     float* __restrict__ CGP, const int* __restrict__ padmeta, int L, int nF, int nFp, int B, int nbF) {
+                     float* __restrict__ CGP, const int* __restrict__ padmeta, int L, int nF, int nFp, int B, int nbF,
+                     int ntab, float* __restrict__ stds_copy, int sumT) {
     __shared__ int s_tab[kMaxLookup];
     int blk = (int)blockIdx.x;
     if (blk < nb_fwd) {
@@ -76,17 +79,24 @@ layer_prepare_kernel(const float2* __restrict__ W, const float* __restrict__ std
         return;
     }
     blk -= nbF;
-    pad_table_block(CG, CGP, padmeta + 2 * (L + 2) + kPadMetaInts * blk);
+    if (blk < ntab) {
+        pad_table_block(CG, CGP, padmeta + 2 * (L + 2) + kPadMetaInts * blk);
+        return;
+    }
+    blk -= ntab;
+    const int c = blk * 256 + (int)threadIdx.x;
+    if (c < sumT) stds_copy[c] = stds[c];
 }
 
-struct SavedAreas { size_t Ag, Fp, CGP, total; };
+struct SavedAreas { size_t stds, Ag, Fp, CGP, total; };
 SavedAreas saved_areas(const cgnet_layer_plan* lp, int B) {
     SavedAreas a{};
     if (!lp->link.ok || B <= 0) return a;
     size_t o = 0;
-    a.Ag = o;  o += align_up(sizeof(float) * lp->link.operand_floats, 256);
-    a.Fp = o;  o += align_up(sizeof(float) * 2 * (size_t)lp->cg->bwd_nFp * B, 256);
-    a.CGP = o; o += align_up(sizeof(float) * (size_t)lp->cg->bwd_cgp_len, 256);
+    a.stds = o; o += align_up(sizeof(float) * (size_t)lp->cg->sumT, 256);   // the stds this batch was normalised with
+    a.Ag = o;   o += align_up(sizeof(float) * lp->link.operand_floats, 256);
+    a.Fp = o;   o += align_up(sizeof(float) * 2 * (size_t)lp->cg->bwd_nFp * B, 256);
+    a.CGP = o;  o += align_up(sizeof(float) * (size_t)lp->cg->bwd_cgp_len, 256);
     a.total = o;
     return a;
 }
@@ -167,6 +177,11 @@ extern "C" size_t cgnet_CGBN_saved_bytes(const cgnet_layer_plan* plan, int B) {
     return plan ? saved_areas(plan, B).total : 0;
 }
 
+extern "C" size_t cgnet_CGBN_saved_stds_bytes(const cgnet_layer_plan* plan, int B) {
+    if (!plan || !plan->link.ok || B <= 0) return 0;
+    return sizeof(float) * (size_t)plan->cg->sumT;          // the copy sits at the start of the area
+}
+
 extern "C" size_t cgnet_CGBN_forward_workspace(const cgnet_layer_plan* plan, int B) {
     if (!plan || B <= 0) return 0;
     return forward_areas(plan, B).total;
@@ -216,13 +231,15 @@ extern "C" int cgnet_CGBN_forward(const cgnet_layer_plan* plan, const float* d_F
     const int nb_gen = save ? (plan->link.npack + 3) / 4 : 0;
     const int nbF = save ? (int)(((size_t)cg->bwd_nFp * B + 255) / 256) : 0;
     const int ntab = save ? cg->nllls : 0;
-    if (nb_fwd + nb_gen + nbF + ntab > 0) {
+    const int nb_std = save && bn ? (cg->sumT + 255) / 256 : 0;
+    if (nb_fwd + nb_gen + nbF + ntab + nb_std > 0) {
         char* sv = (char*)d_saved;
-        CGNET_LAUNCH(layer_prepare_kernel, dim3((unsigned)(nb_fwd + nb_gen + nbF + ntab)), dim3(256), 0, s,
+        CGNET_LAUNCH(layer_prepare_kernel, dim3((unsigned)(nb_fwd + nb_gen + nbF + ntab + nb_std)), dim3(256), 0, s,
                      (const float2*)d_W, bn ? d_stds : nullptr, eps, wmm->d_degs, ndeg, Wp, wmm->wp_blocks, nb_fwd,
                      plan->link.d_gens, plan->link.d_packmap, plan->link.npack, save ? (float*)(sv + sa.Ag) : nullptr,
                      nb_gen, (const float2*)d_F, d_CG, save ? (float2*)(sv + sa.Fp) : nullptr,
-                     save ? (float*)(sv + sa.CGP) : nullptr, cg->d_bwd_padmeta, cg->L, cg->nF, cg->bwd_nFp, B, nbF);
+                     save ? (float*)(sv + sa.CGP) : nullptr, cg->d_bwd_padmeta, cg->L, cg->nF, cg->bwd_nFp, B, nbF, ntab,
+                     save ? (float*)(sv + sa.stds) : nullptr, cg->sumT);
         CGNET_HIP(hipGetLastError());
     }
     return wmm_forward_packed(wmm, d_FF, d_O, Wp, B, ws + fa.opart, s);

@@ -193,6 +193,10 @@ const char* cgnet_CGBN_backward_fused_reason(const cgnet_layer_plan* plan);
  * aligned, or NULL (inference; also when the fused backward is not supported, where the size is 0).
  * d_stds / cnt / eps / flags as in cgnet_FN_WMM_forward. */
 size_t cgnet_CGBN_saved_bytes(const cgnet_layer_plan* plan, int B);
+/* With CGNET_FN_BATCHNORM the area starts with a copy of the stds this batch was normalised with (float,
+ * cgnet_CGBN_saved_stds_bytes(plan, B) bytes = 4 * sum_l t_FF[l]; 0 when nothing is saved): the running values
+ * move on with the next batch, and the weight gradient of this one (cgnet_FN_WMM_backward, d_stds) needs these. */
+size_t cgnet_CGBN_saved_stds_bytes(const cgnet_layer_plan* plan, int B);
 size_t cgnet_CGBN_forward_workspace(const cgnet_layer_plan* plan, int B);
 int cgnet_CGBN_forward(const cgnet_layer_plan* plan, const float* d_F, float* d_FF, float* d_O, const float* d_W,
                        const float* d_CG, int B, float* d_stds, float cnt, float eps, int flags,
