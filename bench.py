@@ -10,7 +10,8 @@ fragments that already reside in HBM.  `roofline` describes the kernel that take
 time inside the timed region (durations from HIP events the library records on the launch
 stream; the timed steps bracket only that kernel, an untimed survey before them brackets every
 kernel for the `kernels` table); `whole_step` prices the complete step against the five
-compulsory passes over the materialised product tensor.  `cpu_baseline` times the CPU oracle (a port of the reference's
+compulsory passes over the materialised product tensor (the default backward skips two of them: it never
+writes grad_FF; `--two-kernel-backward` runs all five).  `cpu_baseline` times the CPU oracle (a port of the reference's
 python path) on a bounded sample of the same workload on the host cores.
 """
 import argparse
@@ -145,8 +146,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--fused-backward", action="store_true",
-                    help="run the layer's backward in one kernel, without grad_FF in memory (default: two kernels)")
+    ap.add_argument("--two-kernel-backward", action="store_true",
+                    help="materialise grad_FF and run the mixing backward and the product backward as two kernels "
+                         "(default: the one-kernel layer backward, which forms grad_FF tile by tile in LDS)")
     ap.add_argument("--cpu-batch", type=int, default=16)
     ap.add_argument("--cpu-repeats", type=int, default=6)
     ap.add_argument("--copy-probe", action="store_true",
@@ -168,8 +170,7 @@ def main():
     lmax, tau, bsz = WORKLOAD["lmax"], WORKLOAD["tau"], WORKLOAD["batch"]
     taus = [tau] * (lmax + 1)
     layer = CG_layers.CGBN_cuda(lmax, taus, taus, batchnorm=True, sparse_flag=False, device=dev)
-    if args.fused_backward:
-        layer.fused_backward = True
+    layer.fused_backward = not args.two_kernel_backward
     t_ff = [int(v) for v in layer.t_FF]
     x, w, go = synthetic(lmax, tau, bsz, t_ff)
     with torch.no_grad():
@@ -249,7 +250,7 @@ def main():
         "cg_backward_kernel": 8 * (bsz * n_ff + 2 * bsz * n_f),
     }
     # the one-kernel layer backward stands for two of the five passes (grad FF written, grad FF read); it is priced
-    # against the bytes those passes would move although it moves neither
+    # against the bytes those passes would move although it moves neither (what it really moves: `traffic`)
     algo["cgbn_backward_fused_kernel"] = algo["wmm_gradff_mfma_kernel"] + algo["cg_backward_hybrid_kernel"]
     measured_traffic, traffic_source = profiled_traffic()
     step_bytes = 8 * (5 * bsz * n_ff + bsz * (3 * n_f + 3 * n_o) + 3 * n_w) + 4 * (2 * sum_t + cg_len)
@@ -282,7 +283,7 @@ def main():
                      "simd_issue": profiled_issue(dominant, d_avg_s * 1e3)},
         "whole_step": {"algorithmic_bytes": step_bytes, "achieved_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
                        "frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        "fused_backward": bool(layer.fused_backward),
+        "fused_backward": bool(layer.fused_backward and layer.native_layer_plan().fused_backward_supported),
         "kernels": kernels,
         "kernels_note": "per-kernel table from %d untimed steps with every launch bracketed by events; "
                         "in the timed steps only the dominant kernel is bracketed" % survey_steps,
