@@ -159,21 +159,27 @@ __device__ __forceinline__ void pack_w_gen_lane(const float2* __restrict__ W, co
         cm = g.chan0 + t2 * tau + t1;
     }
     const float rm = (on && stds && tau) ? fmaxf(eps, stds[g.cumT + cm]) : 1.f;
-    for (int ks = 0; ks < 2 * nkp; ++ks) {
-        const int k = 4 * ks + kk, to = k >> 1;
-        float v = 0.f;
-        if (on && ks < g.nks && to < g.tO) {
-            const float2 w = W[g.cumW + (size_t)to * g.K + c];
-            v = (k & 1) ? w.y : w.x;
-            if (stds) v = v / r;
-            if (tau) {
-                const float2 wm = W[g.cumW + (size_t)to * g.K + cm];
-                float vm = (k & 1) ? wm.y : wm.x;
-                if (stds) vm = vm / rm;
-                v = g.sym < 0 ? v - vm : v + vm;
+    for (int kp = 0; kp < nkp; ++kp) {
+        float pair[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int ks = 2 * kp + h;
+            const int k = 4 * ks + kk, to = k >> 1;
+            float v = 0.f;
+            if (on && ks < g.nks && to < g.tO) {
+                const float2 w = W[g.cumW + (size_t)to * g.K + c];
+                v = (k & 1) ? w.y : w.x;
+                if (stds) v = v / r;
+                if (tau) {
+                    const float2 wm = W[g.cumW + (size_t)to * g.K + cm];
+                    float vm = (k & 1) ? wm.y : wm.x;
+                    if (stds) vm = vm / rm;
+                    v = g.sym < 0 ? v - vm : v + vm;
+                }
             }
+            pair[h] = v;
         }
-        dst[(size_t)(ks >> 1) * 128 + (ks & 1)] = v;
+        *reinterpret_cast<float2*>(dst + (size_t)kp * 128) = make_float2(pair[0], pair[1]);
     }
 }
 

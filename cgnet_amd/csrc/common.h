@@ -151,4 +151,20 @@ __device__ __forceinline__ void stream_store16(void* dst, float a, float b, floa
 // All copies (and loads) this wave has started have landed (vmcnt == 0).
 __device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
+// s_waitcnt vmcnt(n) for a run-time n (the instruction takes an immediate); n above the table waits for all.
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define CGNET_VMCNT(N) case N: __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14)); break;
+    switch (n) {
+        CGNET_VMCNT(1) CGNET_VMCNT(2) CGNET_VMCNT(3) CGNET_VMCNT(4) CGNET_VMCNT(5) CGNET_VMCNT(6) CGNET_VMCNT(7)
+        CGNET_VMCNT(8) CGNET_VMCNT(9) CGNET_VMCNT(10) CGNET_VMCNT(11) CGNET_VMCNT(12) CGNET_VMCNT(13)
+        CGNET_VMCNT(14) CGNET_VMCNT(15) CGNET_VMCNT(16) CGNET_VMCNT(17) CGNET_VMCNT(18) CGNET_VMCNT(19)
+        CGNET_VMCNT(20) CGNET_VMCNT(21) CGNET_VMCNT(22) CGNET_VMCNT(23) CGNET_VMCNT(24) CGNET_VMCNT(25)
+        CGNET_VMCNT(26) CGNET_VMCNT(27) CGNET_VMCNT(28)
+        default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
+    }
+#undef CGNET_VMCNT
+    asm volatile("" ::: "memory");
+}
+
+
 }  // namespace cgnet
