@@ -360,6 +360,8 @@ class CG_woFilter_cuda(nn.Module):
 # CGNET_FUSED_BACKWARD=0: new layers take the two-kernel backward (grad_FF in memory) even where the one-kernel
 # backward is available
 _FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "1")))
+# CGNET_FUSED_INFERENCE=0: new layers materialise FF in evaluation mode too
+_FUSED_INFERENCE = bool(int(os.environ.get("CGNET_FUSED_INFERENCE", "1")))
 
 
 class _CGBN_fused(torch.autograd.Function):
@@ -435,6 +437,10 @@ class CGBN_cuda(nn.Module):
         # grad_FF tensor (B x nFF complex) in memory, where the shapes allow it
         # (cgnet_CGBN_backward_fused_supported); False keeps the two-kernel backward.  Same gradients either way.
         self.fused_backward = _FUSED_BACKWARD
+        # With ``fused``: when no gradient is wanted and the statistics are not updated (evaluation mode, or no fragment
+        # norm), True takes the forward without the product tensor FF (B x nFF complex) in memory, every tile of it mixed
+        # in LDS, where the shapes allow it (cgnet_CGBN_forward_inference_supported); same output up to rounding.
+        self.fused_inference = _FUSED_INFERENCE
         self._layer_plan = None
         self.to(device)
 
@@ -453,9 +459,18 @@ class CGBN_cuda(nn.Module):
                 fs = _straight(fs)
             assert fs.is_cuda
             bn = self.bnWMM
-            new_fs = _CGBN_fused.apply(fs, bn.W, self.native_layer_plan(), self.cg.CGspace, bn.bn_stds, bn.bn_cnt,
-                                       bn._eps_host, bn.training, self.fused_backward)
-            if bn.batchnorm and bn.training:
+            lp = self.native_layer_plan()
+            wants_grad = torch.is_grad_enabled() and (fs.requires_grad or bn.W.requires_grad)
+            updates = bn.batchnorm and bn.training
+            if self.fused_inference and not wants_grad and not updates and lp.inference_forward_supported:
+                B = fs.shape[0]
+                new_fs = torch.empty(B, lp.wmm_plan.nO, 2, device=fs.device, dtype=torch.float)
+                lp.forward_inference(fs.detach().contiguous(), new_fs, bn.W.detach().contiguous(), self.cg.CGspace, B,
+                                     bn.bn_stds, bn._eps_host, BN_FLAG if bn.bn_stds is not None else 0)
+            else:
+                new_fs = _CGBN_fused.apply(fs, bn.W, lp, self.cg.CGspace, bn.bn_stds, bn.bn_cnt, bn._eps_host, bn.training,
+                                           self.fused_backward)
+            if updates:
                 bn.bn_cnt += 1
         else:
             new_fs = self.cg(fs, straight_output=True)

@@ -55,6 +55,11 @@ SIGNATURES = {
     "cgnet_CGBN_backward_fused_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_CGBN_backward_fused": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float,
                                                  ctypes.c_int, _vp, ctypes.c_size_t, _vp, ctypes.c_size_t, _vp]),
+    "cgnet_CGBN_forward_inference_supported": (ctypes.c_int, [_vp]),
+    "cgnet_CGBN_forward_inference_reason": (ctypes.c_char_p, [_vp]),
+    "cgnet_CGBN_forward_inference_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_forward_inference": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float, ctypes.c_int,
+                                                    _vp, ctypes.c_size_t, _vp]),
     "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_forward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_backward_groups": (ctypes.c_int, [_vp]),

@@ -231,6 +231,8 @@ class LayerPlan:
         self._h = h
         self.fused_backward_supported = bool(lib.cgnet_CGBN_backward_fused_supported(self._h))
         self.fused_backward_reason = lib.cgnet_CGBN_backward_fused_reason(self._h).decode("utf-8", "replace")
+        self.inference_forward_supported = bool(lib.cgnet_CGBN_forward_inference_supported(self._h))
+        self.inference_forward_reason = lib.cgnet_CGBN_forward_inference_reason(self._h).decode("utf-8", "replace")
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -267,6 +269,27 @@ class LayerPlan:
                                               0 if saved is None else saved.numel(), _ptr(ws), ws.numel(),
                                               _stream(F.device)))
         return saved
+
+    def forward_inference(self, F, O, W, CG, B, stds, eps, flags):
+        """O = layer(F) without FF in memory (cgnet_CGBN_forward_inference): evaluation mode, no gradient."""
+        cg, wmm = self.cg_plan, self.wmm_plan
+        cg._check_io(F, B)
+        _require_gpu("output", O)
+        _require_gpu("W", W)
+        _require_gpu("CG", CG)
+        if flags & _lib.FN_BATCHNORM:
+            _require_gpu("FN_stds", stds)
+            if stds.numel() != wmm.sum_tFF:
+                raise RuntimeError("FN_stds has %d entries, expected %d" % (stds.numel(), wmm.sum_tFF))
+        else:
+            stds = None
+        if O.numel() != B * wmm.nO * 2 or W.numel() != wmm.nW * 2 or CG.numel() < cg.cg_len:
+            raise RuntimeError("CGBN inference forward: tensor sizes do not match the plans")
+        lib = _lib.load()
+        with torch.cuda.device(F.device):
+            ws = _workspace(lib.cgnet_CGBN_forward_inference_workspace(self._h, int(B)), F.device)
+            _lib.check(lib.cgnet_CGBN_forward_inference(self._h, _ptr(F), _ptr(O), _ptr(W), _ptr(CG), int(B), _ptr(stds),
+                                                        float(eps), int(flags), _ptr(ws), ws.numel(), _stream(F.device)))
 
     def saved_stds(self, saved, B):
         """The float32 view of the stds copy inside a saved-operand tensor (None if it holds none)."""

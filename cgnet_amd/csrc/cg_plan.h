@@ -128,6 +128,37 @@ struct FusedLink {
     size_t lds = 0;                      // LDS bytes of a work-group of the fused kernel
 };
 
+// Fused inference forward (product tile mixed while it lies in LDS; FF never exists): what the mixing half needs to
+// know of a forward task, one entry per cgnet_cg_plan::fwd_tasks entry, in the same order.
+struct FwdMixTask {
+    int aoff;                 // float offset of the task's packed weights: float2 entry [ks * 64 + lane] = (W_re, W_im) / div of
+                              // output channel lane % 16 and the tile's channel 4 ks + lane / 16 (zero past t_O / the tile)
+    int nks;                  // k-steps of four channels over the tile; 0 for a degree without output channels
+    int tO;                   // output channels of degree l
+    int ooff;                 // complex offset of the task's t_O x (2l+1) block inside a sample's partial outputs
+    int cumW, K, c0, cumT;    // degree l: complex offset of its weights, mid channels; the tile's first channel inside the degree;
+                              // first mid channel of the degree among all
+};
+
+struct FwdLaunch {
+    int T;                    // column tiles of 16 values of m of the launch's tasks
+    int sel0, n;              // its tasks: entries [sel0, sel0 + n) of FwdLink::d_sel
+    size_t lds;               // LDS bytes of a work-group
+};
+
+struct FwdLink {
+    bool ok = false;
+    FwdMixTask* d_mix = nullptr;
+    int* d_sel = nullptr;                // indices into the forward tasks, launch by launch
+    std::vector<FwdLaunch> launches;
+    int* d_packmap = nullptr;            // per 64-lane block of the weight packing: task, k-step
+    int* d_red = nullptr;                // [L+2] cumO | [L+1] t_O | [L+2] list begin | per degree the ooff of its tasks, in channel order
+    int npack = 0;
+    size_t a_floats = 0;                 // packed weights, all tasks
+    int opart = 0;                       // complex entries of one sample's partial outputs
+    int nO = 0, L = 0;
+};
+
 }  // namespace cgnet
 
 namespace cgnet {
@@ -181,6 +212,22 @@ __device__ __forceinline__ void pack_w_gen_lane(const float2* __restrict__ W, co
         }
         *reinterpret_cast<float2*>(dst + (size_t)kp * 128) = make_float2(pair[0], pair[1]);
     }
+}
+
+// One lane's share of the packed weights of the fused inference forward (layout: FwdMixTask::aoff).
+__device__ __forceinline__ void pack_w_mix_lane(const float2* __restrict__ W, const float* __restrict__ stds, float eps,
+                                                const FwdMixTask& g, int nch, int ks, int lane, float* __restrict__ Af) {
+    const int to = lane & 15, cl = 4 * ks + (lane >> 4);
+    float2 v = make_float2(0.f, 0.f);
+    if (to < g.tO && cl < nch) {
+        const float2 w = W[g.cumW + (size_t)to * g.K + g.c0 + cl];
+        v = w;
+        if (stds) {
+            const float r = fmaxf(eps, stds[g.cumT + g.c0 + cl]);
+            v = make_float2(w.x / r, w.y / r);
+        }
+    }
+    *reinterpret_cast<float2*>(Af + g.aoff + ((size_t)ks * 64 + lane) * 2) = v;
 }
 
 // Work-group `blk` (256 threads, every thread must call) of the padded fragments: Fp = F with one zero behind

@@ -67,6 +67,10 @@ __device__ __forceinline__ unsigned opaque(unsigned v) {
 
 
 
+__device__ __forceinline__ void lds_barrier() {      // this wave's LDS accesses are complete, then the group's barrier
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ------------------------------------------------------------------------------------ forward
 // The hardware square root (one instruction, error within one ulp).  The statistics use the same
 // rounded modulus in both of their sums, so its last bit does not matter to the variance.
@@ -465,6 +469,164 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
             }
         }
     }
+}
+
+// ---- inference forward of the whole layer: the product tile is mixed while it lies in LDS -------------------------
+// cg_forward_mm_kernel whose tile never leaves for memory: when a sample's tile of a task is complete, the eight waves
+// multiply it with the task's slice of the weights, O_part[to, m] = sum over the tile's channels c of
+// (W[to, c] / div[c]) FF[c, m], on the matrix cores (rows = the up to 16 output channels, columns = T tiles of 16
+// values of m with re / im of a column in one lane, reduction over the channels in steps of four), and what leaves
+// is the task's t_O x (2l+1) partial output, a twelfth of the tile.  cgbn_forward_reduce_kernel adds the partial
+// outputs of a degree's tasks in channel order.  A wave has a role (column tile, share of the reduction steps) and
+// keeps its share of the packed weights in registers for all samples of the group; the shares meet in LDS.
+// Statistics cannot be taken on this route (the mixing needs the stds of the whole batch before the first tile): it
+// serves evaluation mode and layers without fragment norm.
+constexpr int kMixMaxK = 16;                   // reduction steps of one wave (64 channels)
+constexpr int kMixShares = 4;                  // shares of the reduction steps of a column tile: one wave per SIMD
+constexpr size_t kMixShareBytes = 2048;        // a share's 16 x 16 complex partial sums
+
+__host__ __device__ constexpr size_t mix_red_bytes(int T) { return (size_t)T * (kMixShares - 1) * kMixShareBytes; }
+
+template <int T>
+__global__ void __launch_bounds__(kFwdMmThreads, 6)
+cgbn_forward_fused_kernel(const float2* __restrict__ F, const float* __restrict__ CG, const CgTask* __restrict__ tasks,
+                          const FwdMixTask* __restrict__ mix, const int* __restrict__ sel, const float* __restrict__ Af,
+                          float2* __restrict__ Opart, int nF, int B, int samples_per_group, int opart, int lds_bytes) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const UnitPart up = part_major((B + samples_per_group - 1) / samples_per_group);
+    const int unit = sel[up.unit];                                 // the launch's tasks: those with T column tiles
+    const CgTask t = tasks[unit];
+    const FwdMixTask g = mix[unit];
+    const int group = up.part;
+    const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
+    const int P = M2 + 3;
+    const int nch = t.rows * t.tau2;
+    const int nout = nch * M, n1 = t.rows * M1, n2 = t.tau2 * M2;
+    const size_t out_bytes = (8 * (size_t)nout + 15) & ~(size_t)15;
+    const size_t f1_bytes = (8 * (size_t)n1 + 15) & ~(size_t)15;
+    const size_t frag_bytes = fwd_frag_lds(t) + kFwdMmPad;
+    unsigned char* frag = smem + kFwdMmPad;                        // [2][frag_bytes]
+    float2* out = reinterpret_cast<float2*>(frag + 2 * frag_bytes);
+    float* cg = reinterpret_cast<float*>(frag + 2 * frag_bytes + out_bytes);
+    float4* red = reinterpret_cast<float4*>(smem + lds_bytes - mix_red_bytes(T));   // [share - 1][column tile][2][64]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    {
+        float4* z = reinterpret_cast<float4*>(smem);
+        for (int e = tid; e < (lds_bytes >> 4); e += kFwdMmThreads) z[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __syncthreads();                                               // the clearing stores precede every copy
+    auto issue = [&](int b, int par) {
+        const float2* Fb = F + (size_t)b * nF;
+        unsigned char* d1 = frag + par * frag_bytes;
+        unsigned char* d2 = d1 + f1_bytes;
+        dma16<kFwdMmThreads>(Fb + t.offF1, d1, n1 >> 1, tid);
+        if (n1 & 1) dma8(Fb + t.offF1 + (n1 - 1), d1 + 8 * (size_t)(n1 - 1), tid);
+        dma16<kFwdMmThreads>(Fb + t.offF2, d2, n2 >> 1, tid);
+        if (n2 & 1) dma8(Fb + t.offF2 + (n2 - 1), d2 + 8 * (size_t)(n2 - 1), tid);
+    };
+    const int b0 = group * samples_per_group;
+    const int b1 = min(B, b0 + samples_per_group);
+    if (b0 < b1) issue(b0, 0);
+    for (int e = tid; e < M * M2; e += kFwdMmThreads) {            // the table, as in cg_forward_mm_kernel
+        const int r = e / M2, c = e - r * M2;
+        const int m1 = (r - t.l) - (c - t.l2);
+        cg[r * P + c] = (m1 >= -t.l1 && m1 <= t.l1) ? CG[t.cg_off + e] : 0.f;
+    }
+    // role of the wave in the mixing: column tile tcol, share kh of the reduction steps.  Four shares put one wave of
+    // a column tile on every SIMD; with one column tile the other four waves only take part in the product.
+    const int tcol = wave % T, kh = wave / T;
+    const bool mixing = kh < kMixShares && g.nks > 0;
+    const int ks0 = mixing ? (kh * g.nks) / kMixShares : 0, ks1 = mixing ? ((kh + 1) * g.nks) / kMixShares : 0;
+    const int cnt = ks1 - ks0;                                     // <= kMixMaxK (the plan checks)
+    float2 a[kMixMaxK];
+#pragma unroll
+    for (int j = 0; j < kMixMaxK; ++j)
+        a[j] = j < cnt ? reinterpret_cast<const float2*>(Af + g.aoff)[(size_t)(ks0 + j) * 64 + lane] : make_float2(0.f, 0.f);
+    const int i = lane & 15, kk = lane >> 4;
+    const int col = 16 * tcol + i;
+    const unsigned pb_last = lds_addr(out + (nch - 1) * M + min(col, M - 1));
+    const unsigned pb_first = lds_addr(out + (4 * ks0 + kk) * M + min(col, M - 1));
+    const unsigned pb_step = 32u * (unsigned)M;                    // four channels further
+    double dummy1[4] = {0., 0., 0., 0.}, dummy2[4] = {0., 0., 0., 0.};   // the statistics half of fwd_mm_sample's interface
+    int par = 0;
+    for (int b = b0; b < b1; ++b, par ^= 1) {
+        dma_wait();
+        __syncthreads();       // this sample's fragments landed; the previous sample's partial sums have been read
+        if (b + 1 < b1) issue(b + 1, par ^ 1);
+        const float2* f1 = reinterpret_cast<const float2*>(frag + par * frag_bytes);
+        const float2* f2 = reinterpret_cast<const float2*>(frag + par * frag_bytes + f1_bytes);
+        fwd_mm_sample<false>(t, cg, P, f1, f2, out, wave, kFwdMmThreads / 64, lane, dummy1, dummy2);
+        lds_barrier();         // the tile is complete
+        f32x4 xr = {0.f, 0.f, 0.f, 0.f}, yr = xr, xi = xr, yi = xr;
+        if (mixing) {
+            unsigned pb = pb_first;
+#pragma unroll
+            for (int j = 0; j < kMixMaxK; ++j) {
+                if (j < cnt) {
+                    const float2 v = lds_c(min(pb, pb_last), 0);   // channels past the tile's last meet zero weights
+                    pb += pb_step;
+                    xr = mfma4(a[j].x, v.x, xr);
+                    yr = mfma4(a[j].x, v.y, yr);
+                    xi = mfma4(a[j].y, v.x, xi);
+                    yi = mfma4(a[j].y, v.y, yi);
+                }
+            }
+        }
+        // (W_re + i W_im)(x + i y): re = W_re x - W_im y, im = W_re y + W_im x
+        float4 ore = make_float4(xr[0] - yi[0], xr[1] - yi[1], xr[2] - yi[2], xr[3] - yi[3]);
+        float4 oim = make_float4(yr[0] + xi[0], yr[1] + xi[1], yr[2] + xi[2], yr[3] + xi[3]);
+        if (mixing && kh > 0) {
+            float4* mine = red + ((kh - 1) * T + tcol) * 128;
+            mine[lane] = ore;
+            mine[64 + lane] = oim;
+        }
+        lds_barrier();         // the shares have been written; nobody reads the tile any more
+        if (kh == 0 && g.tO > 0) {
+            // the wave that holds share 0 of its column tile adds the others in order and stores the partial output
+            if (g.nks > 0) {
+#pragma unroll
+                for (int k = 1; k < kMixShares; ++k) {
+                    const float4* theirs = red + ((k - 1) * T + tcol) * 128;
+                    const float4 r = theirs[lane], q = theirs[64 + lane];
+                    ore.x += r.x; ore.y += r.y; ore.z += r.z; ore.w += r.w;
+                    oim.x += q.x; oim.y += q.y; oim.z += q.z; oim.w += q.w;
+                }
+            }
+            float2* dst = Opart + (size_t)b * opart + g.ooff + (4 * kk) * M + col;
+            if (col < M) {
+                if (4 * kk + 0 < g.tO) dst[0] = make_float2(ore.x, oim.x);
+                if (4 * kk + 1 < g.tO) dst[M] = make_float2(ore.y, oim.y);
+                if (4 * kk + 2 < g.tO) dst[2 * M] = make_float2(ore.z, oim.z);
+                if (4 * kk + 3 < g.tO) dst[3 * M] = make_float2(ore.w, oim.w);
+            }
+        }
+    }
+}
+
+// O[b][degree l][to][m] = sum of the partial outputs of the degree's tasks, in channel order.
+// meta: [L+2] cumO | [L+1] t_O | [L+2] list begin | the ooff of every task, degree by degree
+__global__ void __launch_bounds__(256)
+cgbn_forward_reduce_kernel(const float2* __restrict__ Opart, float2* __restrict__ O, const int* __restrict__ meta,
+                           int L, int nO, int opart, int B) {
+    __shared__ int s_tab[kMaxLookup];
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int b = (int)(idx / nO), e = (int)(idx % nO);
+    const int* cumO = meta;                 // L+2
+    const int* lbeg = meta + (L + 2) + (L + 1);
+    const int* loff = lbeg + (L + 2);
+    const int lam = lookup_in_group(L + 1, e, [&](int k) { return cumO[k]; }, s_tab);
+    if (idx >= (size_t)B * nO) return;
+    const int rel = e - cumO[lam];
+    const float2* p = Opart + (size_t)b * opart;
+    float2 sum = make_float2(0.f, 0.f);
+#pragma unroll 8
+    for (int k = lbeg[lam]; k < lbeg[lam + 1]; ++k) {
+        const float2 v = p[loff[k] + rel];
+        sum.x += v.x;
+        sum.y += v.y;
+    }
+    O[idx] = sum;
 }
 
 __global__ void __launch_bounds__(256)
@@ -1395,9 +1557,6 @@ cg_backward_hybrid_kernel(const float2* __restrict__ Fp, const float2* __restric
 // in phase 1); the task's own coefficient table and l2 slab, which only phase 2 reads, are copied during its phase 1.
 // Every buffer exists once, which keeps the work-group small enough for three to share a compute unit.  A wave
 // learns about the task after the next one through scalar loads that are in flight for a whole stage.
-__device__ __forceinline__ void lds_barrier() {      // this wave's LDS accesses are complete, then the group's barrier
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
 
 struct FusedCtx {
     const float2* Fp;          // this sample's fragments, rows padded with one zero
@@ -2750,6 +2909,167 @@ int launch_fused_backward(const cgnet_cg_plan* plan, const FusedLink& link, cons
                  (const float2*)d_part1, (const float2*)d_part2, (float2*)d_gF, plan->d_bwd_combine, plan->L,
                  plan->nF, plan->bwd_P2, B);
     CGNET_HIP(hipGetLastError());
+    return CGNET_OK;
+}
+
+}  // namespace cgnet
+
+// ---- fused inference forward: host side -------------------------------------------------------------
+namespace cgnet {
+
+void free_fwd_link(FwdLink* link) {
+    if (!link) return;
+    void* ptrs[] = {link->d_mix, link->d_packmap, link->d_red, link->d_sel};
+    for (void* q : ptrs)
+        if (q) (void)hipFree(q);
+    *link = FwdLink();
+}
+
+int build_fwd_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FwdLink* link) {
+    *link = FwdLink();
+    CGNET_REQUIRE(wmm_plan_degrees(w) == p->L + 1, CGNET_ERR_ARG, "the two plans have different lmax");
+    std::vector<WmmDegInfo> info(p->L + 1);
+    for (int l = 0; l <= p->L; ++l)
+        if (int rc = wmm_plan_degree(w, l, &info[l])) return rc;
+    CGNET_REQUIRE(p->fwd_mm, CGNET_ERR_UNSUPPORTED,
+                  "the fused inference forward needs the matrix-core product (every channel count in 8..16)");
+    CGNET_REQUIRE(p->L <= 15, CGNET_ERR_UNSUPPORTED, "the fused inference forward takes lmax <= 15 (two column tiles of 16 values of m)");
+    for (int l = 0; l <= p->L; ++l)
+        CGNET_REQUIRE(info[l].tO <= 16, CGNET_ERR_UNSUPPORTED, "the fused inference forward needs t_O <= 16 in every degree");
+    const int nt = (int)p->fwd_tasks.size();
+    std::vector<FwdMixTask> mix(nt);
+    std::vector<int> map;
+    std::vector<std::vector<std::pair<int, int>>> per_l(p->L + 1);       // (first channel, ooff) of every task of a degree
+    size_t aoff = 0;
+    int ooff = 0;
+    for (int k = 0; k < nt; ++k) {
+        const CgTask& t = p->fwd_tasks[k];
+        const WmmDegInfo& d = info[t.l];
+        const int nch = t.rows * t.tau2, M = 2 * t.l + 1;
+        CGNET_REQUIRE(nch <= 4 * 64, CGNET_ERR_UNSUPPORTED, "a product tile of %d channels exceeds the mixing registers", nch);
+        FwdMixTask g{};
+        g.aoff = (int)aoff;
+        g.nks = d.tO > 0 ? (nch + 3) / 4 : 0;
+        g.tO = d.tO;
+        g.ooff = ooff;
+        g.cumW = d.cumW;
+        g.K = d.K;
+        g.c0 = t.chan0 - p->cumT[t.l];
+        g.cumT = d.cumT;
+        mix[k] = g;
+        for (int ks = 0; ks < g.nks; ++ks) { map.push_back(k); map.push_back(ks); }
+        aoff += (size_t)g.nks * 128;
+        CGNET_REQUIRE(aoff < (1u << 30), CGNET_ERR_UNSUPPORTED, "packed weights of the fused forward exceed 2^30 floats");
+        if (d.tO > 0) per_l[t.l].push_back(std::make_pair(g.c0, ooff));
+        ooff += d.tO * M;
+    }
+    std::vector<int> red;
+    for (int l = 0; l <= p->L; ++l) red.push_back(info[l].cumO);
+    const int nO = info[p->L].cumO + info[p->L].tO * (2 * p->L + 1);
+    red.push_back(nO);
+    for (int l = 0; l <= p->L; ++l) red.push_back(info[l].tO);
+    int run = 0;
+    for (int l = 0; l <= p->L; ++l) { red.push_back(run); run += (int)per_l[l].size(); }
+    red.push_back(run);
+    for (int l = 0; l <= p->L; ++l) {
+        std::sort(per_l[l].begin(), per_l[l].end());                      // channel order: the order the mixing kernel adds in
+        for (const auto& e : per_l[l]) red.push_back(e.second);
+    }
+    FwdLink tmp;
+    auto upload = [](const void* src, size_t bytes, void** dst) -> int {
+        if (bytes == 0) return CGNET_OK;
+        CGNET_HIP(hipMalloc(dst, bytes));
+        CGNET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return CGNET_OK;
+    };
+    int rc = upload(mix.data(), sizeof(FwdMixTask) * mix.size(), (void**)&tmp.d_mix);
+    if (!rc) rc = upload(map.data(), sizeof(int) * map.size(), (void**)&tmp.d_packmap);
+    if (!rc) rc = upload(red.data(), sizeof(int) * red.size(), (void**)&tmp.d_red);
+    // one launch per (LDS class, number of column tiles of 16 values of m), over the class's tasks of that kind in the
+    // class's order (by work)
+    std::vector<int> sel;
+    size_t lds_max[3] = {0, 0, 0};
+    for (size_t k = 0; k + 1 < p->fwd_class_begin.size(); ++k)
+        for (int T = 1; T <= 2; ++T) {
+            FwdLaunch fl{};
+            fl.T = T;
+            fl.sel0 = (int)sel.size();
+            for (int i = p->fwd_class_begin[k]; i < p->fwd_class_begin[k + 1]; ++i)
+                if ((2 * p->fwd_tasks[i].l + 1 + 15) / 16 == T) sel.push_back(i);
+            fl.n = (int)sel.size() - fl.sel0;
+            fl.lds = p->fwd_class_lds[k] + mix_red_bytes(T);
+            if (fl.n == 0) continue;
+            lds_max[T] = std::max(lds_max[T], fl.lds);
+            tmp.launches.push_back(fl);
+        }
+    if (!rc) rc = upload(sel.data(), sizeof(int) * sel.size(), (void**)&tmp.d_sel);
+    if (!rc && std::max(lds_max[1], lds_max[2]) > kMaxLds) {
+        set_error("the fused inference forward would need %zu bytes of LDS per work-group (limit %zu)",
+                  std::max(lds_max[1], lds_max[2]), kMaxLds);
+        rc = CGNET_ERR_UNSUPPORTED;
+    }
+    if (!rc && lds_max[1]) rc = raise_dynamic_lds((const void*)cgbn_forward_fused_kernel<1>, lds_max[1]);
+    if (!rc && lds_max[2]) rc = raise_dynamic_lds((const void*)cgbn_forward_fused_kernel<2>, lds_max[2]);
+    if (rc) {
+        free_fwd_link(&tmp);
+        return rc;
+    }
+    tmp.npack = (int)(map.size() / 2);
+    tmp.a_floats = aoff;
+    tmp.opart = ooff;
+    tmp.nO = nO;
+    tmp.L = p->L;
+    tmp.ok = true;
+    *link = tmp;
+    return CGNET_OK;
+}
+
+// the tasks' packed weights: four (task, k-step) blocks of 64 lanes per work-group
+__global__ void __launch_bounds__(256)
+pack_w_mix_kernel(const float2* __restrict__ W, const float* __restrict__ stds, float eps, const CgTask* __restrict__ tasks,
+                  const FwdMixTask* __restrict__ mix, const int* __restrict__ map, int npack, float* __restrict__ Af) {
+    const int pair = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+    if (pair >= npack) return;
+    const int k = map[2 * pair];
+    pack_w_mix_lane(W, stds, eps, mix[k], tasks[k].rows * tasks[k].tau2, map[2 * pair + 1], threadIdx.x & 63, Af);
+}
+
+int launch_pack_w_mix(const cgnet_cg_plan* p, const FwdLink& link, const float* d_W, const float* d_stds, float eps, float* d_Af,
+                      hipStream_t s) {
+    if (link.npack > 0) {
+        CGNET_LAUNCH(pack_w_mix_kernel, dim3((unsigned)((link.npack + 3) / 4)), dim3(256), 0, s, (const float2*)d_W, d_stds, eps,
+                     p->d_fwd_tasks, link.d_mix, link.d_packmap, link.npack, d_Af);
+        CGNET_HIP(hipGetLastError());
+    }
+    return CGNET_OK;
+}
+
+int launch_forward_fused(const cgnet_cg_plan* p, const FwdLink& link, const float* d_F, const float* d_CG, const float* d_Af,
+                         float* d_Opart, float* d_O, int B, hipStream_t s) {
+    CGNET_REQUIRE(link.ok, CGNET_ERR_UNSUPPORTED, "the fused inference forward does not take this pair of plans");
+    const int ntasks = (int)p->fwd_tasks.size();
+    const int spg = samples_per_group_for(B, ntasks);
+    const int ngroups = (B + spg - 1) / spg;
+    CGNET_REQUIRE((long long)ntasks * ngroups < (1LL << 31), CGNET_ERR_UNSUPPORTED,
+                  "%d tasks x %d sample groups exceed the grid limit", ntasks, ngroups);
+    for (const FwdLaunch& fl : link.launches) {
+        if (fl.T == 1) {
+            CGNET_LAUNCH(cgbn_forward_fused_kernel<1>, dim3((unsigned)(fl.n * ngroups)), dim3(kFwdMmThreads), fl.lds, s,
+                         (const float2*)d_F, d_CG, p->d_fwd_tasks, link.d_mix, link.d_sel + fl.sel0, d_Af, (float2*)d_Opart,
+                         p->nF, B, spg, link.opart, (int)fl.lds);
+        } else {
+            CGNET_LAUNCH(cgbn_forward_fused_kernel<2>, dim3((unsigned)(fl.n * ngroups)), dim3(kFwdMmThreads), fl.lds, s,
+                         (const float2*)d_F, d_CG, p->d_fwd_tasks, link.d_mix, link.d_sel + fl.sel0, d_Af, (float2*)d_Opart,
+                         p->nF, B, spg, link.opart, (int)fl.lds);
+        }
+        CGNET_HIP(hipGetLastError());
+    }
+    const size_t n = (size_t)link.nO * B;
+    if (n > 0) {
+        CGNET_LAUNCH(cgbn_forward_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const float2*)d_Opart,
+                     (float2*)d_O, link.d_red, link.L, link.nO, link.opart, B);
+        CGNET_HIP(hipGetLastError());
+    }
     return CGNET_OK;
 }
 

@@ -36,4 +36,13 @@ int launch_fused_backward(const cgnet_cg_plan* p, const FusedLink& link, const f
                           const float* d_Fp, const float* d_CGP, float* d_Bg, float* d_part1, float* d_part2,
                           float* d_gF, int B, hipStream_t s);
 
+// ---- fused inference forward (cg_product.hip)
+int build_fwd_link(const cgnet_cg_plan* p, const cgnet_wmm_plan* w, FwdLink* link);
+void free_fwd_link(FwdLink* link);
+int launch_pack_w_mix(const cgnet_cg_plan* p, const FwdLink& link, const float* d_W, const float* d_stds, float eps, float* d_Af,
+                      hipStream_t s);
+// product tiles mixed in LDS + the sum of the tasks' partial outputs; d_Opart: link.opart * B complex entries
+int launch_forward_fused(const cgnet_cg_plan* p, const FwdLink& link, const float* d_F, const float* d_CG, const float* d_Af,
+                         float* d_Opart, float* d_O, int B, hipStream_t s);
+
 }  // namespace cgnet

@@ -13,6 +13,8 @@ struct cgnet_layer_plan {
     const cgnet_wmm_plan* wmm = nullptr;
     cgnet::FusedLink link;
     char reason[512] = "";       // why the fused backward does not take this layer ("" if it does)
+    cgnet::FwdLink fwd;
+    char fwd_reason[512] = "";   // why the fused inference forward does not take it
 };
 
 namespace cgnet {
@@ -153,6 +155,14 @@ extern "C" int cgnet_layer_plan_create(cgnet_layer_plan** plan, const cgnet_cg_p
     } else if (rc != CGNET_OK) {
         return rc;
     }
+    const int rc2 = build_fwd_link(cg_plan, wmm_plan, &p->fwd);
+    if (rc2 == CGNET_ERR_UNSUPPORTED) {
+        std::strncpy(p->fwd_reason, cgnet_last_error(), sizeof(p->fwd_reason) - 1);
+        clear_error();
+    } else if (rc2 != CGNET_OK) {
+        free_fused_link(&p->link);
+        return rc2;
+    }
     *plan = p.release();
     return CGNET_OK;
 }
@@ -160,6 +170,7 @@ extern "C" int cgnet_layer_plan_create(cgnet_layer_plan** plan, const cgnet_cg_p
 extern "C" int cgnet_layer_plan_destroy(cgnet_layer_plan* plan) {
     clear_error();
     if (!plan) return CGNET_OK;
+    free_fwd_link(&plan->fwd);
     free_fused_link(&plan->link);
     delete plan;
     return CGNET_OK;
@@ -289,4 +300,41 @@ extern "C" int cgnet_CGBN_backward_fused(const cgnet_layer_plan* plan, const flo
     }
     return launch_fused_backward(cg, plan->link, d_gO, Ag, Fp, CGP, (float*)(ws + ba.Bg), (float*)(ws + ba.own.part1),
                                  (float*)(ws + ba.own.part2), d_gF, B, s);
+}
+
+// ---- inference forward without FF ---------------------------------------------------------------------
+extern "C" int cgnet_CGBN_forward_inference_supported(const cgnet_layer_plan* plan) { return plan && plan->fwd.ok ? 1 : 0; }
+
+extern "C" const char* cgnet_CGBN_forward_inference_reason(const cgnet_layer_plan* plan) {
+    return plan ? plan->fwd_reason : "no plan";
+}
+
+extern "C" size_t cgnet_CGBN_forward_inference_workspace(const cgnet_layer_plan* plan, int B) {
+    if (!plan || !plan->fwd.ok || B <= 0) return 0;
+    return align_up(sizeof(float) * plan->fwd.a_floats, 256) + align_up(sizeof(float) * 2 * (size_t)plan->fwd.opart * B, 256);
+}
+
+extern "C" int cgnet_CGBN_forward_inference(const cgnet_layer_plan* plan, const float* d_F, float* d_O, const float* d_W,
+                                            const float* d_CG, int B, const float* d_stds, float eps, int flags,
+                                            void* d_workspace, size_t workspace_bytes, void* stream) {
+    clear_error();
+    CGNET_REQUIRE(plan, CGNET_ERR_ARG, "plan is NULL");
+    CGNET_REQUIRE(B >= 0, CGNET_ERR_ARG, "B=%d is negative", B);
+    if (B == 0 || plan->wmm->nO == 0) return CGNET_OK;
+    CGNET_REQUIRE(plan->fwd.ok, CGNET_ERR_UNSUPPORTED, "%s", plan->fwd_reason);
+    const bool bn = flags & CGNET_FN_BATCHNORM;
+    CGNET_REQUIRE(!(flags & CGNET_FN_UPDATE_STD), CGNET_ERR_ARG,
+                  "the inference forward cannot update the running stds (they depend on the whole batch's product)");
+    CGNET_REQUIRE(!bn || d_stds, CGNET_ERR_ARG, "batch-norm flag set but d_stds is NULL");
+    CGNET_REQUIRE(d_O && (plan->cg->nF == 0 || d_F) && (plan->wmm->nW == 0 || d_W) && (plan->cg->nFF == 0 || d_CG), CGNET_ERR_ARG,
+                  "null device pointer");
+    const size_t need = cgnet_CGBN_forward_inference_workspace(plan, B);
+    CGNET_REQUIRE(d_workspace && workspace_bytes >= need, CGNET_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed",
+                  workspace_bytes, need);
+    CGNET_REQUIRE(((uintptr_t)d_workspace & 15) == 0, CGNET_ERR_ARG, "workspace must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    float* Af = (float*)d_workspace;
+    float* Opart = (float*)((char*)d_workspace + align_up(sizeof(float) * plan->fwd.a_floats, 256));
+    if (int rc = launch_pack_w_mix(plan->cg, plan->fwd, d_W, bn ? d_stds : nullptr, eps, Af, s)) return rc;
+    return launch_forward_fused(plan->cg, plan->fwd, d_F, d_CG, Af, Opart, d_O, B, s);
 }

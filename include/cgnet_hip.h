@@ -216,6 +216,22 @@ int cgnet_CGBN_backward_fused(const cgnet_layer_plan* plan, const float* d_F, fl
                               const void* d_saved, size_t saved_bytes,
                               void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* O = layer(F) for inference, without the product tensor FF (B x nFF complex) ever existing in memory: every tile
+ * of it is mixed with its slice of W / max(eps, stds) on the matrix cores while it lies in LDS, and what leaves the
+ * product kernel is a partial output per kept triple (t_O x (2l+1) values for a tile of t_F[l1] t_F[l2] x (2l+1)); a second
+ * kernel adds the partial outputs of a degree in channel order.  Same result as cgnet_CGBN_forward up to the order of
+ * the additions.  The running stds cannot be updated on this route (CGNET_FN_UPDATE_STD is refused): normalising a
+ * batch with its own statistics needs the whole batch's product first.  It serves CGBN_cuda in evaluation mode
+ * (CGNet/CG_layers.py:313-318 with self.training false) and layers without fragment norm, when no gradient is
+ * wanted.  Supported where the product runs on the matrix cores (every input channel count in 8..16), lmax <= 15
+ * and t_O <= 16; cgnet_CGBN_forward_inference_supported / _reason as for the fused backward.  Allocates nothing. */
+int cgnet_CGBN_forward_inference_supported(const cgnet_layer_plan* plan);
+const char* cgnet_CGBN_forward_inference_reason(const cgnet_layer_plan* plan);
+size_t cgnet_CGBN_forward_inference_workspace(const cgnet_layer_plan* plan, int B);
+int cgnet_CGBN_forward_inference(const cgnet_layer_plan* plan, const float* d_F, float* d_O, const float* d_W,
+                                 const float* d_CG, int B, const float* d_stds, float eps, int flags,
+                                 void* d_workspace, size_t workspace_bytes, void* stream);
+
 /* ---- measurement hooks (no counterpart in the reference, which times nothing) ------------ */
 
 /* With timing enabled every kernel launch of this library is bracketed by two HIP events

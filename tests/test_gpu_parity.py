@@ -641,6 +641,47 @@ def test_fused_backward_equals_two_kernel_backward(dev, monkeypatch, lmax, tin, 
         check_layer_step(dev, mod, ora, twin, w64, x64, go.double().cpu())
 
 
+def _inference_cases():
+    return _fused_backward_cases(10, 57)[:10] + [(11, [12] * 12, [12] * 12, 3, False, True, 100),
+                                                 (15, [16] * 16, [16] * 16, 1, True, True, 101),
+                                                 (12, [8, 16, 9, 12, 10, 8, 13, 16, 8, 11, 12, 9, 14],
+                                                  [3, 0, 16, 12, 1, 7, 0, 5, 16, 2, 9, 4, 6], 2, False, True, 102),
+                                                 (9, [10] * 10, [5] * 10, 9, False, False, 103)]
+
+
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _inference_cases())
+def test_inference_forward_without_product_tensor(dev, lmax, tin, tout, bsz, sparse, bn, k):
+    """Evaluation mode without a gradient: the forward that never holds FF in memory (every product tile mixed in LDS,
+    partial outputs per triple added in channel order) against the oracle, and against the route through FF."""
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=700 + k)
+    lp = mod.native_layer_plan()
+    assert lp.inference_forward_supported, lp.inference_forward_reason
+    mod.eval()
+    ora.training = twin.training = False
+    x64 = rand_straight(tin, bsz, seed=800 + k)
+    want = OL.join_straight(ora.forward(x64, w64))
+    tw = OL.join_straight(twin.forward(x64.float(), w64.float()))
+    x = x64.float().to(dev)
+    from cgnet_amd import _lib
+    lib = _lib.load()
+    with torch.no_grad():
+        lib.cgnet_profile_reset()
+        lib.cgnet_profile_enable(1)
+        out = mod(x, straight_output=True)
+        torch.cuda.synchronize()
+        lib.cgnet_profile_enable(0)
+        names = set(_lib.kernel_times())
+        mod.fused_inference = False
+        out_ff = mod(x, straight_output=True)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    if n_o:
+        assert "cgbn_forward_fused_kernel" in names and "wmm_forward_kernel" not in names, names   # the route that was meant
+    assert_close(out, want, "inference forward without FF", tw)
+    assert_close(out_ff, want, "inference forward through FF", tw)
+    if bn:
+        assert mod.bnWMM.bn_cnt == 1.0 and torch.equal(mod.bnWMM.bn_stds.cpu(), torch.from_numpy(twin.stds_flat()))
+
+
 def test_invalid_table_slots_are_never_used(dev):
     """Slots of the flat table whose m1 = m - m2 is no index of degree l1 carry no coefficient; the reference's
     kernels never read them (cudaCG_sparse.cu:164,243).  Here the matrix-core kernels walk over them, so every
