@@ -345,8 +345,23 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
         unsigned pa = opaque(a_row + 8u * (unsigned)(m - lo + l1 - kk));
         unsigned pb = opaque(b_row + 8u * (unsigned)(lo + l2 + kk));
         unsigned pc = opaque(c_lane + 4u * (unsigned)(mm * P + lo + l2));
-        f32x4 dre = {0.f, 0.f, 0.f, 0.f}, dim = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < nsteps; ++s) {
+        // the first step starts from constant zero accumulators (every m has at least one step: the plan only
+        // admits triples that obey the triangle rule)
+        f32x4 dre, dim;
+        {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            const float c = lds_f(pc)[0];
+            const float2 fa = lds_c(pa, 0), fb = lds_c(pb, 0);
+            pa -= 32u;
+            pb += 32u;
+            pc += 16u;
+            const float ar = c * fa.x, ai = c * fa.y, nai = -ai;
+            dre = mfma4(ar, fb.x, zero);
+            dim = mfma4(ar, fb.y, zero);
+            dre = mfma4(nai, fb.y, dre);
+            dim = mfma4(ai, fb.x, dim);
+        }
+        for (int s = 1; s < nsteps; ++s) {
             const float c = lds_f(pc)[0];
             const float2 fa = lds_c(pa, 0), fb = lds_c(pb, 0);
             pa -= 32u;
@@ -359,10 +374,15 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
             dim = mfma4(ai, fb.x, dim);
         }
         if (i < tau2) {
-            float2* o = out + (4 * kk * tau2 + i) * M + mm;
+            // re and im go out as two 4-byte writes (one two-address LDS instruction): an 8-byte write would first
+            // copy the pair into adjacent registers
+            float* o = reinterpret_cast<float*>(out + (4 * kk * tau2 + i) * M + mm);
 #pragma unroll
             for (int v = 0; v < 4; ++v)
-                if (4 * kk + v < rows) o[v * tau2 * M] = make_float2(dre[v], dim[v]);
+                if (4 * kk + v < rows) {
+                    o[2 * v * tau2 * M] = dre[v];
+                    o[2 * v * tau2 * M + 1] = dim[v];
+                }
         }
         if (STATS) {
             // both sums run over the same rounded |z| in double (see cg_forward_kernel); lanes past the task's
