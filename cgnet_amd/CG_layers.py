@@ -362,6 +362,9 @@ class CG_woFilter_cuda(nn.Module):
 _FUSED_BACKWARD = bool(int(os.environ.get("CGNET_FUSED_BACKWARD", "1")))
 # CGNET_FUSED_INFERENCE=0: new layers materialise FF in evaluation mode too
 _FUSED_INFERENCE = bool(int(os.environ.get("CGNET_FUSED_INFERENCE", "1")))
+# CGNET_COMPACT_FF=0: the product tensor inside a layer keeps the reference's layout (both orderings of every channel
+# pair of a diagonal triple) also where nothing outside the layer's own kernels reads it
+_COMPACT_FF = bool(int(os.environ.get("CGNET_COMPACT_FF", "1")))
 
 
 class _CGBN_fused(torch.autograd.Function):
@@ -378,10 +381,14 @@ class _CGBN_fused(torch.autograd.Function):
         B = Fs.shape[0]
         dev = Fs.device
         flags = (BN_FLAG if bn_stds is not None else 0) | (UPDATESTD_FLAG if training else 0)
-        FF = torch.empty(B, cg_plan.nFF, 2, device=dev, dtype=torch.float)
-        out = torch.empty(B, wmm_plan.nO, 2, device=dev, dtype=torch.float)
         need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         ctx.fused_backward = bool(fused_backward) and layer_plan.fused_backward_supported
+        # With the one-kernel backward nothing reads FF but the mixing and the weight gradient, and the layer keeps
+        # it in its compact layout (one channel per pair of a diagonal triple) where it has one.
+        if ctx.fused_backward and layer_plan.compact_supported and _COMPACT_FF:
+            flags |= _lib.LAYER_COMPACT_FF
+        FF = torch.empty(B, layer_plan.internal_nFF(flags), 2, device=dev, dtype=torch.float)
+        out = torch.empty(B, wmm_plan.nO, 2, device=dev, dtype=torch.float)
         # the operands of the one-kernel backward are prepared beside those of the mixing forward, in the same launch
         saved_ops = layer_plan.forward(Fs, FF, out, W, CG, B, bn_stds, float(bn_cnt), float(bn_eps), flags,
                                        save=ctx.fused_backward and ctx.needs_input_grad[0])
@@ -404,12 +411,14 @@ class _CGBN_fused(torch.autograd.Function):
         need_F, need_W = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         grad_W = torch.empty_like(W) if need_W else None
         grad_F = torch.empty_like(Fs) if need_F else None
-        if need_F and ctx.fused_backward:
+        if ctx.fused_backward:
             # The gradient with respect to FF never exists in memory: the product's backward forms every tile of
             # it in LDS from grad_output and the weights.  The weight gradient needs FF, not grad_FF.
             if need_W:
-                wmm_plan.backward(grad_output, None, grad_W, FF, W, ctx.B, stds, ctx.eps, ctx.flags)
-            ctx.layer_plan.backward_fused(Fs, grad_F, grad_output, W, CG, ctx.B, stds, ctx.eps, ctx.flags, saved_ops)
+                ctx.layer_plan.backward_gradw(grad_output, FF, grad_W, ctx.B, stds, ctx.eps, ctx.flags)
+            if need_F:
+                ctx.layer_plan.backward_fused(Fs, grad_F, grad_output, W, CG, ctx.B, stds, ctx.eps,
+                                              ctx.flags & (BN_FLAG | UPDATESTD_FLAG), saved_ops)
             return grad_F, grad_W, None, None, None, None, None, None, None
         grad_FF = torch.empty_like(FF) if need_F else None
         if need_F or need_W:

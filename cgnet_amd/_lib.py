@@ -12,6 +12,7 @@ LIB_PATH = os.environ.get("CGNET_HIP_LIBRARY") or os.path.join(_HERE, "csrc", "l
 
 OK, ERR_ARG, ERR_HIP, ERR_WORKSPACE, ERR_UNSUPPORTED = 0, -1, -2, -3, -4
 FN_BATCHNORM, FN_UPDATE_STD = 0x1, 0x2
+LAYER_COMPACT_FF = 0x4     # cgnet_CGBN_forward / _backward_gradw: product tensor in the layer's compact layout
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -60,6 +61,11 @@ SIGNATURES = {
     "cgnet_CGBN_forward_inference_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int]),
     "cgnet_CGBN_forward_inference": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float, ctypes.c_int,
                                                     _vp, ctypes.c_size_t, _vp]),
+    "cgnet_CGBN_compact_supported": (ctypes.c_int, [_vp]),
+    "cgnet_CGBN_internal_nFF": (ctypes.c_size_t, [_vp, ctypes.c_int]),
+    "cgnet_CGBN_backward_gradw_workspace": (ctypes.c_size_t, [_vp, ctypes.c_int, ctypes.c_int]),
+    "cgnet_CGBN_backward_gradw": (ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_float, ctypes.c_int,
+                                                 _vp, ctypes.c_size_t, _vp]),
     "cgnet_cg_plan_backward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_forward_lds": (ctypes.c_size_t, [_vp]),
     "cgnet_cg_plan_backward_groups": (ctypes.c_int, [_vp]),

@@ -233,6 +233,12 @@ class LayerPlan:
         self.fused_backward_reason = lib.cgnet_CGBN_backward_fused_reason(self._h).decode("utf-8", "replace")
         self.inference_forward_supported = bool(lib.cgnet_CGBN_forward_inference_supported(self._h))
         self.inference_forward_reason = lib.cgnet_CGBN_forward_inference_reason(self._h).decode("utf-8", "replace")
+        # the layer may keep its product tensor in a compact layout (one channel per pair of a diagonal triple)
+        self.compact_supported = bool(lib.cgnet_CGBN_compact_supported(self._h))
+
+    def internal_nFF(self, flags):
+        """Complex entries per sample of the product tensor ``forward`` writes with these flags."""
+        return int(_lib.load().cgnet_CGBN_internal_nFF(self._h, int(flags)))
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -255,7 +261,7 @@ class LayerPlan:
                 raise RuntimeError("FN_stds has %d entries, expected %d" % (stds.numel(), wmm.sum_tFF))
         else:
             stds = None
-        if (FF.numel() != B * cg.nFF * 2 or O.numel() != B * wmm.nO * 2 or W.numel() != wmm.nW * 2
+        if (FF.numel() != B * self.internal_nFF(flags) * 2 or O.numel() != B * wmm.nO * 2 or W.numel() != wmm.nW * 2
                 or CG.numel() < cg.cg_len):
             raise RuntimeError("CGBN forward: tensor sizes do not match the plans")
         lib = _lib.load()
@@ -320,3 +326,23 @@ class LayerPlan:
                                                      _ptr(stds), float(eps), int(flags), _ptr(saved),
                                                      0 if saved is None else saved.numel(), _ptr(ws), ws.numel(),
                                                      _stream(F.device)))
+
+    def backward_gradw(self, gO, FF, gW, B, stds, eps, flags):
+        """gW of the layer from gO and the product tensor ``forward`` wrote with the same flags
+        (cgnet_CGBN_backward_gradw)."""
+        wmm = self.wmm_plan
+        _require_gpu("grad_out", gO)
+        _require_gpu("FF", FF)
+        _require_gpu("grad_W", gW)
+        if flags & _lib.FN_BATCHNORM:
+            _require_gpu("FN_stds", stds)
+        else:
+            stds = None
+        if (gO.numel() != B * wmm.nO * 2 or FF.numel() != B * self.internal_nFF(flags) * 2 or gW.numel() != wmm.nW * 2):
+            raise RuntimeError("layer weight gradient: tensor sizes do not match the plans")
+        gO, FF = _aligned16(gO), _aligned16(FF)
+        lib = _lib.load()
+        with torch.cuda.device(gO.device):
+            ws = _workspace(lib.cgnet_CGBN_backward_gradw_workspace(self._h, int(B), int(flags)), gO.device)
+            _lib.check(lib.cgnet_CGBN_backward_gradw(self._h, _ptr(gO), _ptr(FF), _ptr(gW), int(B), _ptr(stds), float(eps),
+                                                     int(flags), _ptr(ws), ws.numel(), _stream(gO.device)))

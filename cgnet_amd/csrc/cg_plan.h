@@ -19,6 +19,9 @@ struct CgTask {
     int chan0;            // index over all mid channels (all degrees) of the tile's first channel
     int nT1, nT2, TI, TJ; // forward register tiling: rows = nT1 x TI (strided), tau2 = nT2 x TJ
     int bTI[2], bRW[2];   // backward, per slot: output channels per thread, lanes sharing one output
+    int sym;              // matrix-core forward only: 1 = the tile of a diagonal triple (l1 = l2, all rows) is stored in
+                          // its compact form, the channels (t1 <= t2, t2) column after column; offFF / chan0 then count compact
+                          // channels.  0 in every table of a product plan (the reference's layout).
 };
 
 // Backward, register-resident scheme: one work-group per (sample, unit), a unit being the

@@ -331,6 +331,13 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
     const int M = 2 * l + 1, M1 = 2 * l1 + 1, M2 = 2 * l2 + 1;
     const int rows = t.rows, tau2 = t.tau2;
     const int i = lane & 15, kk = lane >> 4;
+    // Channel of the result (row r = 4 kk + v, column i): r tau2 + i.  In the compact tile of a diagonal triple only
+    // the columns i >= r exist, column after column: i (i + 1) / 2 + r -- so that in both layouts the four results
+    // of a lane lie a constant number of channels apart.
+    const int r0 = 4 * kk;
+    const int chan_lane = t.sym ? i * (i + 1) / 2 + r0 : r0 * tau2 + i;
+    const int chan_step = t.sym ? 1 : tau2;
+    const int last_row = t.sym ? min(rows - 1, i) : rows - 1;     // rows r0 + v <= last_row are stored
     // rows / channels past the end repeat the last one (their results are not stored)
     const unsigned a_row = lds_addr(f1 + min(i, rows - 1) * M1);
     const unsigned b_row = lds_addr(f2 + min(i, tau2 - 1) * M2);
@@ -376,12 +383,12 @@ __device__ __forceinline__ void fwd_mm_sample(const CgTask& t, const float* __re
         if (i < tau2) {
             // re and im go out as two 4-byte writes (one two-address LDS instruction): an 8-byte write would first
             // copy the pair into adjacent registers
-            float* o = reinterpret_cast<float*>(out + (4 * kk * tau2 + i) * M + mm);
+            float* o = reinterpret_cast<float*>(out + chan_lane * M + mm);
 #pragma unroll
             for (int v = 0; v < 4; ++v)
-                if (4 * kk + v < rows) {
-                    o[2 * v * tau2 * M] = dre[v];
-                    o[2 * v * tau2 * M + 1] = dim[v];
+                if (r0 + v <= last_row) {
+                    o[2 * v * chan_step * M] = dre[v];
+                    o[2 * v * chan_step * M + 1] = dim[v];
                 }
         }
         if (STATS) {
@@ -409,9 +416,11 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
     const int group = up.part;
     const int M = 2 * t.l + 1, M1 = 2 * t.l1 + 1, M2 = 2 * t.l2 + 1;
     const int P = M2 + 3;
-    const int nch = t.rows * t.tau2;
+    // channels the tile holds in memory: all rows x tau2, or the upper triangle of a compact diagonal tile (the LDS
+    // is laid out for the full tile either way)
+    const int nch = t.sym ? t.rows * (t.rows + 1) / 2 : t.rows * t.tau2;
     const int nout = nch * M, n1 = t.rows * M1, n2 = t.tau2 * M2;
-    const size_t out_bytes = (8 * (size_t)nout + 15) & ~(size_t)15;
+    const size_t out_bytes = (8 * (size_t)t.rows * t.tau2 * M + 15) & ~(size_t)15;
     const size_t f1_bytes = (8 * (size_t)n1 + 15) & ~(size_t)15;
     const size_t frag_bytes = fwd_frag_lds(t) + kFwdMmPad;          // one buffer and the pad behind it
     unsigned char* frag = smem + kFwdMmPad;                        // [2][frag_bytes]
@@ -480,7 +489,15 @@ cg_forward_mm_kernel(const float2* __restrict__ F, float2* __restrict__ FF, cons
             __syncthreads();
             // thread -> channel (row r, column c) of the task; its value lies at lane (r / 4) * 16 + c, slot r % 4
             for (int ch = tid; ch < nch; ch += kFwdMmThreads) {
-                const int r = ch / t.tau2, c = ch - r * t.tau2;
+                int r = ch / t.tau2, c = ch - r * t.tau2;
+                if (t.sym) {                                       // compact tile: column c holds the rows 0 .. c
+                    c = 0;
+                    r = ch;
+                    while (r > c) {
+                        r -= c + 1;
+                        ++c;
+                    }
+                }
                 const int src = (r & 3) * 64 + (r >> 2) * 16 + c;
                 double sum = 0.;
 #pragma unroll
@@ -2089,6 +2106,7 @@ extern "C" int cgnet_cg_plan_create(cgnet_cg_plan** plan, int L, const int* h_t_
                 t.TJ = (tau2 + t.nT2 - 1) / t.nT2;
                 t.bTI[0] = t.bTI[1] = 1;
                 t.bRW[0] = t.bRW[1] = 1;
+                t.sym = 0;
                 out->push_back(t);
             }
         }
@@ -2558,7 +2576,12 @@ extern "C" int cgnet_cg_plan_channels(const cgnet_cg_plan* plan, int* h_t_FF, in
 }
 
 int cgnet::cg_launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF, const float* d_CG, int B,
-                          double* d_part, int spg, hipStream_t s) {
+                          double* d_part, int spg, hipStream_t s, const CgTask* d_tasks, int nFF, int sumT) {
+    if (!d_tasks) {
+        d_tasks = p->d_fwd_tasks;
+        nFF = p->nFF;
+        sumT = p->sumT;
+    }
     const int ntasks = (int)p->fwd_tasks.size();
     if (ntasks == 0 || B == 0) return CGNET_OK;
     const int ngroups = (B + spg - 1) / spg;
@@ -2568,12 +2591,11 @@ int cgnet::cg_launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_
         const int t0 = p->fwd_class_begin[k], nt = p->fwd_class_begin[k + 1] - t0;
         if (p->fwd_mm) {
             CGNET_LAUNCH(cg_forward_mm_kernel, dim3((unsigned)(nt * ngroups)), dim3(kFwdMmThreads), p->fwd_class_lds[k], s,
-                         (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
-                         p->sumT, (int)p->fwd_class_lds[k]);
+                         (const float2*)d_F, (float2*)d_FF, d_CG, d_tasks + t0, p->nF, nFF, B, spg, d_part, sumT,
+                         (int)p->fwd_class_lds[k]);
         } else {
             CGNET_LAUNCH(cg_forward_kernel, dim3((unsigned)(nt * ngroups)), dim3(kThreads), p->fwd_class_lds[k], s,
-                         (const float2*)d_F, (float2*)d_FF, d_CG, p->d_fwd_tasks + t0, p->nF, p->nFF, B, spg, d_part,
-                         p->sumT);
+                         (const float2*)d_F, (float2*)d_FF, d_CG, d_tasks + t0, p->nF, nFF, B, spg, d_part, sumT);
         }
         CGNET_HIP(hipGetLastError());
     }

@@ -998,6 +998,25 @@ int wmm_plan_degree(const cgnet_wmm_plan* plan, int l, WmmDegInfo* info) {
 }  // namespace cgnet
 
 static int gradw_chunks(int B) { return (B + kGradWChunk - 1) / kGradWChunk; }
+
+namespace cgnet {
+size_t wmm_gradw_part_bytes(const cgnet_wmm_plan* plan, int B) {
+    return sizeof(float) * 2 * (size_t)plan->nW * gradw_chunks(B);
+}
+int wmm_gradw_raw(const cgnet_wmm_plan* plan, const float* d_gO, const float* d_FF, float* d_part, int B, int* nchunks_out,
+                  hipStream_t s) {
+    // equal chunks of at most kGradWChunk samples; the kernel derives the number of chunks from their size
+    const int spc = (B + gradw_chunks(B) - 1) / gradw_chunks(B);
+    const int nchunks = (B + spc - 1) / spc;             // <= gradw_chunks(B), what the partial area holds
+    const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
+    CGNET_LAUNCH(wmm_gradw_kernel, dim3(grid_1d(plan->gw_units.size(), nchunks)), dim3(kThreads), lds, s,
+                 (const float2*)d_gO, (const float2*)d_FF, (float2*)d_part, plan->d_degs, plan->d_gw_units, B, spc,
+                 plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
+    CGNET_HIP(hipGetLastError());
+    *nchunks_out = nchunks;
+    return CGNET_OK;
+}
+}  // namespace cgnet
 static size_t gff_operand_bytes(const cgnet_wmm_plan* plan) {
     return plan->gff_mfma ? sizeof(float) * 64 * (size_t)plan->ap_blocks : sizeof(float) * 2 * (size_t)plan->nW;
 }
@@ -1033,14 +1052,8 @@ extern "C" int cgnet_FN_WMM_backward(const cgnet_wmm_plan* plan, const float* d_
             CGNET_HIP(hipGetLastError());
         } else {
             CGNET_REQUIRE(d_gO && d_FF, CGNET_ERR_ARG, "null device pointer");
-            // equal chunks of at most kGradWChunk samples; the kernel derives the number of chunks from their size
-            const int spc = (B + gradw_chunks(B) - 1) / gradw_chunks(B);
-            const int nchunks = (B + spc - 1) / spc;             // <= gradw_chunks(B), what the workspace holds
-            const size_t lds = sizeof(float2) * 2 * ((size_t)plan->gw_ff_cap + plan->gw_go_cap);
-            CGNET_LAUNCH(wmm_gradw_kernel, dim3(grid_1d(plan->gw_units.size(), nchunks)), dim3(kThreads), lds, s,
-                               (const float2*)d_gO, (const float2*)d_FF, gw_part, plan->d_degs, plan->d_gw_units, B,
-                               spc, plan->nFF, plan->nO, plan->nW, plan->gw_ff_cap, plan->gw_go_cap);
-            CGNET_HIP(hipGetLastError());
+            int nchunks = 0;
+            if (int rc = wmm_gradw_raw(plan, d_gO, d_FF, (float*)gw_part, B, &nchunks, s)) return rc;
             CGNET_LAUNCH(wmm_gradw_finish_kernel, dim3((plan->nW + 255) / 256), dim3(256), 0, s,
                                (const float2*)gw_part, bn ? d_stds : nullptr, eps, plan->d_degs, ndeg,
                                (float2*)d_gW, plan->nW, nchunks);

@@ -13,11 +13,19 @@ size_t wmm_forward_opart_bytes(const cgnet_wmm_plan* plan, int B);    // partial
 int wmm_forward_packed(const cgnet_wmm_plan* plan, const float* d_FF, float* d_O, const float* d_Wp, int B,
                        void* d_opart, hipStream_t s);
 
+// raw weight-gradient sums  sum_{b in chunk, m} gO conj(FF)  per chunk of samples: d_part[chunk][nW] complex
+// (wmm_gradw_part_bytes bytes); *nchunks = chunks written.  The caller adds them and divides by the stds.
+size_t wmm_gradw_part_bytes(const cgnet_wmm_plan* plan, int B);
+int wmm_gradw_raw(const cgnet_wmm_plan* plan, const float* d_gO, const float* d_FF, float* d_part, int B, int* nchunks,
+                  hipStream_t s);
+
 // ---- cg_product.hip
 int samples_per_group_for(int B, int ntasks);
 // the product kernels of one call; d_part != nullptr: also the per-group partial statistics [group][sumT][2]
+// d_tasks: another table of the plan's forward tasks, in the same order, whose tiles lie elsewhere in the product
+// tensor (nFF complex entries and sumT channels per sample); nullptr = the plan's own
 int cg_launch_forward(const cgnet_cg_plan* p, const float* d_F, float* d_FF, const float* d_CG, int B, double* d_part,
-                      int spg, hipStream_t s);
+                      int spg, hipStream_t s, const CgTask* d_tasks = nullptr, int nFF = 0, int sumT = 0);
 // Per-task metadata of the fused layer backward for this pair of plans, on the current device.  link->ok says
 // whether the fused kernel takes the pair; when it does not, the return code is CGNET_ERR_UNSUPPORTED and
 // cgnet_last_error() names the reason.

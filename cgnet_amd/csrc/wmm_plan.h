@@ -71,9 +71,15 @@ __device__ __forceinline__ float updated_std(float old, double s1, double s2, do
 // four per lane = (k-step 0 | 1) x (W_re | W_im) of W[rc*16+row][kb*8 + 4*step + kk] / div with
 // lane = 16*kk + row.  Thread `idx` writes the four floats of one lane (two weights, one 16-byte store).  Every thread
 // of the group must call (one barrier inside).
+// With a channel map the plan `degs` counts compact mid channels while W and stds keep the layout of `full`: compact
+// channel c of a degree stands for the channel cmap[cumT + c].x (index over all degrees of the full layout) and, where
+// cmap[..].y >= 0, also for that mirror channel, whose product entries are (-1)^l times the first one's; its weight
+// is then the sum of the two normalised weights.
 __device__ __forceinline__ void pack_w_forward_thread(const float2* __restrict__ W, const float* __restrict__ stds,
                                                       float eps, const WmmDeg* __restrict__ degs, int ndeg,
-                                                      float* __restrict__ Wp, int total_blocks, int idx, int* s_tab) {
+                                                      float* __restrict__ Wp, int total_blocks, int idx, int* s_tab,
+                                                      const WmmDeg* __restrict__ full = nullptr,
+                                                      const int2* __restrict__ cmap = nullptr) {
     const int blk = idx >> 4;                                     // 64-float block of the packed array
     const int di = lookup_in_group(ndeg, blk, [&](int k) { return degs[k].wp_base; }, s_tab);
     if (blk >= total_blocks) return;
@@ -86,18 +92,49 @@ __device__ __forceinline__ void pack_w_forward_thread(const float2* __restrict__
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (to < d.tO) {
         const int c0 = kb * 8 + kk, c1 = c0 + 4;
-        const float2* wrow = W + d.cumW + (size_t)to * d.K;
-        float2 w0 = make_float2(0.f, 0.f), w1 = w0;
-        float r0 = 1.f, r1 = 1.f;
-        if (c0 < d.K) {
-            w0 = wrow[c0];
-            if (stds) r0 = fmaxf(eps, stds[d.cumT + c0]);
+        if (cmap) {
+            const WmmDeg f = full[di];
+            const float2* wrow = W + f.cumW + (size_t)to * f.K - f.cumT;     // indexed by the channel over all degrees
+            const float sgn = (d.l & 1) ? -1.f : 1.f;
+            auto folded = [&](int c) {
+                float2 w = make_float2(0.f, 0.f);
+                if (c < d.K) {
+                    const int2 m = cmap[d.cumT + c];
+                    w = wrow[m.x];
+                    if (stds) {
+                        const float r = fmaxf(eps, stds[m.x]);
+                        w.x /= r;
+                        w.y /= r;
+                    }
+                    if (m.y >= 0) {
+                        float2 u = wrow[m.y];
+                        if (stds) {
+                            const float r = fmaxf(eps, stds[m.y]);
+                            u.x /= r;
+                            u.y /= r;
+                        }
+                        w.x += sgn * u.x;
+                        w.y += sgn * u.y;
+                    }
+                }
+                return w;
+            };
+            const float2 w0 = folded(c0), w1 = folded(c1);
+            v = make_float4(w0.x, w0.y, w1.x, w1.y);
+        } else {
+            const float2* wrow = W + d.cumW + (size_t)to * d.K;
+            float2 w0 = make_float2(0.f, 0.f), w1 = w0;
+            float r0 = 1.f, r1 = 1.f;
+            if (c0 < d.K) {
+                w0 = wrow[c0];
+                if (stds) r0 = fmaxf(eps, stds[d.cumT + c0]);
+            }
+            if (c1 < d.K) {
+                w1 = wrow[c1];
+                if (stds) r1 = fmaxf(eps, stds[d.cumT + c1]);
+            }
+            v = stds ? make_float4(w0.x / r0, w0.y / r0, w1.x / r1, w1.y / r1) : make_float4(w0.x, w0.y, w1.x, w1.y);
         }
-        if (c1 < d.K) {
-            w1 = wrow[c1];
-            if (stds) r1 = fmaxf(eps, stds[d.cumT + c1]);
-        }
-        v = stds ? make_float4(w0.x / r0, w0.y / r0, w1.x / r1, w1.y / r1) : make_float4(w0.x, w0.y, w1.x, w1.y);
     }
     reinterpret_cast<float4*>(Wp)[idx] = v;
 }

@@ -232,6 +232,27 @@ int cgnet_CGBN_forward_inference(const cgnet_layer_plan* plan, const float* d_F,
                                  const float* d_CG, int B, const float* d_stds, float eps, int flags,
                                  void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* Compact product tensor.  For a triple with l1 = l2 the reference keeps both orderings (t1, t2), (t2, t1) of every
+ * channel pair (CGNet/CG_layers.py:253-262), and FF[(t2, t1)] = (-1)^l FF[(t1, t2)]: a ninth of FF at L=11, tau=12 is
+ * redundant.  Inside the layer FF is invisible to the user, so with CGNET_LAYER_COMPACT_FF in `flags`
+ * cgnet_CGBN_forward writes only the channels (t1 <= t2, t2) of such triples (cgnet_CGBN_internal_nFF(plan, flags)
+ * complex entries per sample instead of nFF), mixes them with the two weights of a pair added up, and updates the
+ * stds of both channels of a pair from the pair's one set of sums.  O, the stds and the saved operands are the same
+ * as without the flag up to rounding.  A compact FF serves exactly two consumers: cgnet_CGBN_backward_gradw (below)
+ * and nothing else -- cgnet_FN_WMM_backward and cgnet_sparse_backward expect the reference's layout -- so the flag
+ * belongs with the one-kernel backward, which reads no FF.  cgnet_CGBN_compact_supported: 1 where the one-kernel
+ * backward is supported, the product runs on the matrix cores and some diagonal triple is a single forward task.
+ * gW of the layer (what cgnet_FN_WMM_backward(d_gFF = NULL) returns in d_gW) from gO and the FF that
+ * cgnet_CGBN_forward wrote with the same `flags` (without the compact flag this IS cgnet_FN_WMM_backward).
+ * d_stds: the stds the batch was normalised with (reference layout).  Allocates nothing. */
+#define CGNET_LAYER_COMPACT_FF 0x4
+int cgnet_CGBN_compact_supported(const cgnet_layer_plan* plan);
+size_t cgnet_CGBN_internal_nFF(const cgnet_layer_plan* plan, int flags);
+size_t cgnet_CGBN_backward_gradw_workspace(const cgnet_layer_plan* plan, int B, int flags);
+int cgnet_CGBN_backward_gradw(const cgnet_layer_plan* plan, const float* d_gO, const float* d_FF, float* d_gW, int B,
+                              const float* d_stds, float eps, int flags, void* d_workspace, size_t workspace_bytes,
+                              void* stream);
+
 /* ---- measurement hooks (no counterpart in the reference, which times nothing) ------------ */
 
 /* With timing enabled every kernel launch of this library is bracketed by two HIP events

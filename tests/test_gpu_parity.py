@@ -602,8 +602,11 @@ def test_fused_backward_equals_two_kernel_backward(dev, monkeypatch, lmax, tin, 
     input gradient and the weight gradient, in training mode.  Without the fold of the diagonal triples
     (CGNET_DIAG_FOLD=0 when the layer plan is made) the two routes agree bit for bit; with it (the default) the triples
     with l1 = l2 are summed in another order (symmetrised tile, one slot's arithmetic), so the input gradients agree to
-    rounding.  The small cases are also held against the oracle."""
+    rounding.  The product tensor keeps the reference's layout on both routes here (the compact layout, which only the
+    one-kernel route can use, has a test of its own below).  The small cases are also held against the oracle."""
     monkeypatch.setenv("CGNET_DIAG_FOLD", "1" if fold else "0")
+    from cgnet_amd import CG_layers
+    monkeypatch.setattr(CG_layers, "_COMPACT_FF", False)
     mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=400 + k)
     lp = mod.native_layer_plan()
     if not lp.fused_backward_supported:
@@ -638,6 +641,52 @@ def test_fused_backward_equals_two_kernel_backward(dev, monkeypatch, lmax, tin, 
                 mod.bnWMM.bn_stds.copy_(stds0)
         mod.bnWMM.bn_cnt = 1.0
         mod.fused_backward = True
+        check_layer_step(dev, mod, ora, twin, w64, x64, go.double().cpu())
+
+
+@pytest.mark.parametrize("training", [True, False])
+@pytest.mark.parametrize("lmax,tin,tout,bsz,sparse,bn,k", _fused_backward_cases(10, 77))
+def test_compact_product_tensor(dev, monkeypatch, lmax, tin, tout, bsz, sparse, bn, k, training):
+    """Inside a layer with the one-kernel backward the product tensor keeps one channel per pair (t1, t2), (t2, t1) of a
+    diagonal triple (their entries differ by the sign (-1)^l): output, running stds, weight gradient and input gradient
+    against the same layer with the reference's layout (rounding apart: the two weights of a pair are added before
+    the mixing instead of their products after it), and the small cases against the oracle."""
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tin, tout, sparse, bn, seed=900 + k)
+    lp = mod.native_layer_plan()
+    if not lp.compact_supported:
+        pytest.skip("no compact layout for this layer")
+    from cgnet_amd import _lib
+    assert lp.internal_nFF(_lib.LAYER_COMPACT_FF) < lp.internal_nFF(0) == lp.cg_plan.nFF
+    mod.train(training)
+    x64 = rand_straight(tin, bsz, seed=1000 + k)
+    n_o = sum(t * (2 * l + 1) for l, t in enumerate(tout))
+    go = randn32((bsz, n_o, 2), torch.Generator().manual_seed(1100 + k)).float().to(dev)
+    stds0 = mod.bnWMM.bn_stds.detach().clone() if bn else None
+    res = []
+    from cgnet_amd import CG_layers
+    for compact in (False, True):
+        monkeypatch.setattr(CG_layers, "_COMPACT_FF", compact)
+        mod.bnWMM.bn_cnt = 1.0
+        if bn:
+            with torch.no_grad():
+                mod.bnWMM.bn_stds.copy_(stds0)
+        mod.bnWMM.W.grad = None
+        x = x64.float().to(dev).requires_grad_(True)
+        out = mod(x, straight_output=True)
+        out.backward(go)
+        res.append((out.detach().clone(), x.grad.clone(), mod.bnWMM.W.grad.clone() if mod.bnWMM.W.numel() else None,
+                    mod.bnWMM.bn_stds.detach().clone() if bn else None))
+    for name, a, b in zip(("output", "input gradient", "weight gradient", "running stds"), res[0], res[1]):
+        if a is None:
+            continue
+        scale = float(a.abs().max())
+        err = float((a - b).abs().max())
+        assert err <= 3e-5 * scale + 1e-30, "%s differs: max %.3e at scale %.3e" % (name, err, scale)
+    if lmax <= 8 and training:
+        if bn:
+            with torch.no_grad():
+                mod.bnWMM.bn_stds.copy_(stds0)
+        mod.bnWMM.bn_cnt = 1.0
         check_layer_step(dev, mod, ora, twin, w64, x64, go.double().cpu())
 
 
