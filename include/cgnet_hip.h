@@ -233,7 +233,7 @@ int cgnet_CGBN_forward_inference(const cgnet_layer_plan* plan, const float* d_F,
                                  void* d_workspace, size_t workspace_bytes, void* stream);
 
 /* Compact product tensor.  For a triple with l1 = l2 the reference keeps both orderings (t1, t2), (t2, t1) of every
- * channel pair (CGNet/CG_layers.py:253-262), and FF[(t2, t1)] = (-1)^l FF[(t1, t2)]: a ninth of FF at L=11, tau=12 is
+ * channel pair (CGNet/CG_layers.py:253-262), and FF[(t2, t1)] = (-1)^l FF[(t1, t2)]: 8 % of FF at L=11, tau=12 is
  * redundant.  Inside the layer FF is invisible to the user, so with CGNET_LAYER_COMPACT_FF in `flags`
  * cgnet_CGBN_forward writes only the channels (t1 <= t2, t2) of such triples (cgnet_CGBN_internal_nFF(plan, flags)
  * complex entries per sample instead of nFF), mixes them with the two weights of a pair added up, and updates the
