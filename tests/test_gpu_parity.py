@@ -682,6 +682,15 @@ def test_compact_product_tensor(dev, monkeypatch, lmax, tin, tout, bsz, sparse, 
         scale = float(a.abs().max())
         err = float((a - b).abs().max())
         assert err <= 3e-5 * scale + 1e-30, "%s differs: max %.3e at scale %.3e" % (name, err, scale)
+    if res[1][2] is not None:
+        # only the weights want a gradient: the compact tensor still serves the weight gradient, bit for bit the same
+        mod.bnWMM.bn_cnt = 1.0
+        if bn:
+            with torch.no_grad():
+                mod.bnWMM.bn_stds.copy_(stds0)
+        mod.bnWMM.W.grad = None
+        mod(x64.float().to(dev), straight_output=True).backward(go)
+        assert torch.equal(mod.bnWMM.W.grad, res[1][2])
     if lmax <= 8 and training:
         if bn:
             with torch.no_grad():
