@@ -150,7 +150,7 @@ def main():
                     help="materialise grad_FF and run the mixing backward and the product backward as two kernels "
                          "(default: the one-kernel layer backward, which forms grad_FF tile by tile in LDS)")
     ap.add_argument("--cpu-batch", type=int, default=16)
-    ap.add_argument("--cpu-repeats", type=int, default=6)
+    ap.add_argument("--cpu-repeats", type=int, default=8)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 768 MiB read + 768 MiB write elementwise kernel before the warm-up "
                          "(a known-size reference for calibrating hardware byte counters)")
