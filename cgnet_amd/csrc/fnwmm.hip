@@ -253,7 +253,7 @@ wmm_forward_kernel(const float2* __restrict__ FF, const float* __restrict__ Wp, 
     const WmmDeg d = degs[u.deg];
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave index, held in a scalar register
-    const int b_first = (up.part * 4 + w) * d.G;
+    const int b_first = (up.part * (int)(blockDim.x >> 6) + w) * d.G;   // a group is one wave or four
     if (b_first >= B) return;                                     // wave-uniform; the kernel has no barrier
     unsigned char* ring = smem + (size_t)w * depth * stage_bytes;
 #define CGNET_FWD_T(T_) wmm_forward_wave<T_>(FF, Wp, out, d, u, B, nFF, nO, b_first, ring, depth, stage_bytes, lane)
@@ -955,23 +955,27 @@ int wmm_forward_packed(const cgnet_wmm_plan* plan, const float* d_FF, float* d_O
         CGNET_LAUNCH(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)out, n);
         CGNET_HIP(hipGetLastError());
     }
+    // Work-groups of one wave: the waves do not cooperate, and a group that is one wave leaves no LDS idle beside a
+    // short last group of samples and lets the grid drain wave by wave (CGNET_WMM_FWD_WPG=4: four waves a group).
+    static const int wpg = [] { const char* e = getenv("CGNET_WMM_FWD_WPG"); return e && atoi(e) == 4 ? 4 : 1; }();
     int ygroups = 1;
     for (const WmmDeg& d : plan->degs)
-        if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + 4 * d.G - 1) / (4 * d.G));
+        if (d.K > 0 && d.tO > 0) ygroups = std::max(ygroups, (B + wpg * d.G - 1) / (wpg * d.G));
     CGNET_REQUIRE(ygroups <= 65535, CGNET_ERR_UNSUPPORTED, "B=%d too large", B);
     // the LDS-direct copies address the first 64 KB of a group's LDS
-    const int depth = (int)std::min<size_t>(kFwdDepth, (64 * 1024) / (4 * (size_t)plan->fwd_stage_cap));
+    static const int want_depth = [] { const char* e = getenv("CGNET_WMM_FWD_DEPTH"); return e ? atoi(e) : kFwdDepth; }();
+    const int depth = (int)std::min<size_t>(want_depth, (64 * 1024) / (wpg * (size_t)plan->fwd_stage_cap));
     CGNET_REQUIRE(depth >= 2, CGNET_ERR_UNSUPPORTED, "forward stage of %d bytes does not fit the LDS ring", plan->fwd_stage_cap);
-    const size_t lds = 4 * (size_t)depth * plan->fwd_stage_cap;
+    const size_t lds = wpg * (size_t)depth * plan->fwd_stage_cap;
     if (plan->fwd_units_small > 0) {
-        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3(grid_1d(plan->fwd_units_small, ygroups)), dim3(kThreads), lds, s,
+        CGNET_LAUNCH(wmm_forward_kernel<3>, dim3(grid_1d(plan->fwd_units_small, ygroups)), dim3(64 * wpg), lds, s,
                      (const float2*)d_FF, Wp, out, plan->d_degs, plan->d_fwd_units, B, plan->nFF, plan->nO,
                      plan->fwd_stage_cap, depth, ygroups);
         CGNET_HIP(hipGetLastError());
     }
     if ((int)plan->fwd_units.size() > plan->fwd_units_small) {
         CGNET_LAUNCH(wmm_forward_kernel<6>, dim3(grid_1d(plan->fwd_units.size() - plan->fwd_units_small, ygroups)),
-                     dim3(kThreads), lds, s, (const float2*)d_FF, Wp, out, plan->d_degs,
+                     dim3(64 * wpg), lds, s, (const float2*)d_FF, Wp, out, plan->d_degs,
                      plan->d_fwd_units + plan->fwd_units_small, B, plan->nFF, plan->nO, plan->fwd_stage_cap, depth,
                      ygroups);
         CGNET_HIP(hipGetLastError());
