@@ -1046,6 +1046,21 @@ def test_full_size_layer_config3_against_oracle(dev):
     assert mod.bnWMM.bn_cnt == 1.0
 
 
+@pytest.mark.timeout(900)
+def test_full_size_layer_config3_training_step(dev):
+    """The benchmark's own step -- configuration 3 (L=11, tau=12, B=100) in training mode, forward and backward on the
+    default route (statistics of the whole batch taken in the product kernel, compact product tensor, one-kernel
+    backward) -- against the oracle run on the whole batch at once: output, updated running stds, input gradient and
+    weight gradient."""
+    lmax, tau, bsz = 11, [12] * 12, 100
+    mod, ora, twin, w64 = build_layer_pair(dev, lmax, tau, tau, False, True, seed=4)
+    assert mod.native_layer_plan().fused_backward_supported and mod.native_layer_plan().compact_supported
+    x64 = rand_straight(tau, bsz, seed=43)
+    go64 = randn32((bsz, 1728, 2), torch.Generator().manual_seed(45))
+    check_layer_step(dev, mod, ora, twin, w64, x64, go64)
+    assert mod.bnWMM.bn_cnt == 2.0
+
+
 @pytest.mark.parametrize("sparse", [True, False])
 def test_full_size_properties_config4(dev, sparse):
     """benchmark configuration 4 (L=15, tau=16, B=64, MST and default triples): CG product forward + backward."""
