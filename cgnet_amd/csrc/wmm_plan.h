@@ -94,20 +94,20 @@ __device__ __forceinline__ void pack_w_forward_thread(const float2* __restrict__
         const int c0 = kb * 8 + kk, c1 = c0 + 4;
         if (cmap) {
             const WmmDeg f = full[di];
-            const float2* wrow = W + f.cumW + (size_t)to * f.K - f.cumT;     // indexed by the channel over all degrees
+            const float2* wrow = W + f.cumW + (size_t)to * f.K;             // the row; cmap holds channels over all degrees
             const float sgn = (d.l & 1) ? -1.f : 1.f;
             auto folded = [&](int c) {
                 float2 w = make_float2(0.f, 0.f);
                 if (c < d.K) {
                     const int2 m = cmap[d.cumT + c];
-                    w = wrow[m.x];
+                    w = wrow[m.x - f.cumT];
                     if (stds) {
                         const float r = fmaxf(eps, stds[m.x]);
                         w.x /= r;
                         w.y /= r;
                     }
                     if (m.y >= 0) {
-                        float2 u = wrow[m.y];
+                        float2 u = wrow[m.y - f.cumT];
                         if (stds) {
                             const float r = fmaxf(eps, stds[m.y]);
                             u.x /= r;
